@@ -1,0 +1,148 @@
+/*
+ * moe_i8.h — C-ABI of the gfx950 INT8 W8A8 fused-MoE library (libmoe_i8.so).
+ *
+ * Every entry point takes raw device pointers, plain sizes and a HIP stream
+ * (passed as void*).  The library never allocates or frees device memory,
+ * never synchronises and never touches any stream but the one it is given, so
+ * every call can be recorded into a HIP graph.  The caller owns all buffers,
+ * including the workspace.
+ *
+ * Return value: 0 on success, a negative MOE_I8_E* code otherwise; the text of
+ * the last error of the calling thread is available from moe_i8_last_error().
+ *
+ * The reference (prime-rl) holds no FFI for this path: its rollout engine
+ * reaches these operations through vLLM 0.28.0 (reference pyproject.toml:58),
+ * selected by the `quantization` pass-through
+ * (packages/prime-rl-configs/src/prime_rl/configs/inference.py:108-109).  Each
+ * declaration below names the vLLM operation it replaces and the closest
+ * statement of the same semantics that is in the reference tree.
+ */
+#ifndef MOE_I8_H_
+#define MOE_I8_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOE_I8_OK 0
+#define MOE_I8_EINVAL (-1)     /* bad argument (null pointer, size, alignment, limit) */
+#define MOE_I8_EWORKSPACE (-2) /* workspace or output capacity too small */
+#define MOE_I8_ELAUNCH (-3)    /* HIP reported an error at launch */
+#define MOE_I8_EUNSUPPORTED (-4)
+
+#define MOE_I8_MAX_EXPERTS 1024
+
+/* Activation element types accepted by the quantiser / produced by the GEMMs. */
+#define MOE_I8_DTYPE_BF16 0
+
+/* GEMM kernel families; MOE_I8_GEMM_AUTO picks by rows-per-expert. */
+#define MOE_I8_GEMM_AUTO 0
+#define MOE_I8_GEMM_STREAM 1 /* weights streamed global->registers, 16-row MFMA sub-tiles (decode) */
+#define MOE_I8_GEMM_TILE 2   /* LDS-staged double-buffered tiles, 32x32x32 MFMA (prefill) */
+
+int moe_i8_version(void);
+const char* moe_i8_last_error(void);
+
+/* Capacity rules shared with the Python host: sorted_token_ids needs
+ * min(P + E*(B-1), P*B) entries (P = number of (token, expert) pairs) and
+ * expert_ids needs ceil(that / B). */
+int64_t moe_i8_sorted_capacity(int64_t num_pairs, int num_experts, int block_size);
+int64_t moe_i8_align_workspace_bytes(int64_t num_pairs, int num_experts, int block_size);
+
+/*
+ * Replaces vLLM `moe_align_block_size(topk_ids, block_size, num_experts)`
+ * (csrc/moe/moe_align_sum_kernels.cu).  In-tree semantics: stable expert sort
+ * trainer/distributed/token_dispatcher.py:139-145, per-expert padding :107-121.
+ * topk_ids int32 [num_pairs] -> sorted_token_ids int32 [sorted_cap] (flat pair
+ * index, ascending inside each expert segment, unused slots = num_pairs),
+ * expert_ids int32 [expert_cap] (unused blocks = -1), num_tokens_post_padded
+ * int32 [1].  Ids outside [0, num_experts) are ignored.
+ */
+int moe_i8_align_block_size(const int32_t* topk_ids, int64_t num_pairs, int num_experts,
+                            int block_size, int32_t* sorted_token_ids, int64_t sorted_cap,
+                            int32_t* expert_ids, int64_t expert_cap,
+                            int32_t* num_tokens_post_padded, void* workspace,
+                            int64_t workspace_bytes, void* stream);
+
+/*
+ * Replaces vLLM `per_token_quant_int8(x)` (quantization/utils/int8_utils.py);
+ * in-tree analogue trainer/models/kernels/fp8_utils.py:186-201.
+ * x [*, cols] (dtype code, row stride in elements) -> q int8 [rows, cols] and
+ * scale fp32 [rows].  With gather != NULL output row r quantises input row
+ * gather[r] / gather_div; a source row >= src_rows yields a zero row.
+ */
+int moe_i8_quant_rows(const void* x, int dtype, int64_t src_rows, int64_t cols, int64_t row_stride,
+                      const int32_t* gather, int gather_div, int64_t rows, int8_t* q, float* scale,
+                      void* stream);
+
+/*
+ * Replaces vLLM `fused_moe_kernel` (gate_up GEMM, use_int8_w8a8, per-channel) +
+ * `silu_and_mul` (csrc/activation_kernels.cu).  In-tree semantics: grouped GEMM
+ * contract tests/unit/train/models/test_moe.py:60-66; gate-then-up stacking
+ * trainer/models/layers/moe.py:146-148; activation trainer/models/layers/activations.py:29-34.
+ * x_q int8 [M, H], a_scale fp32 [M], w1 int8 [E, 2I, H], w1_scale fp32 [E, 2I]
+ * -> act bf16 [num_pairs, I], row t = pair t (token t / top_k).
+ */
+int moe_i8_gemm_gate_up_silu(const int8_t* x_q, const float* a_scale, const int8_t* w1,
+                             const float* w1_scale, const int32_t* sorted_token_ids,
+                             const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
+                             int64_t num_pairs, int top_k, int num_experts, int hidden, int inter,
+                             int block_size, int64_t sorted_cap, void* act_out, int variant,
+                             void* stream);
+
+/*
+ * Replaces vLLM `fused_moe_kernel` (down GEMM, top_k=1, MUL_ROUTED_WEIGHT).
+ * In-tree semantics: weight applied after the experts in fp32 then cast,
+ * trainer/distributed/token_dispatcher.py:159-160.
+ * h_q int8 [num_pairs, I], a_scale fp32 [num_pairs], w2 int8 [E, H, I],
+ * w2_scale fp32 [E, H], topk_weights fp32 [num_pairs] -> out bf16 [num_pairs, H].
+ */
+int moe_i8_gemm_down(const int8_t* h_q, const float* a_scale, const int8_t* w2,
+                     const float* w2_scale, const float* topk_weights,
+                     const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                     const int32_t* num_tokens_post_padded, int64_t num_pairs, int num_experts,
+                     int hidden, int inter, int block_size, int64_t sorted_cap, void* out,
+                     int variant, void* stream);
+
+/*
+ * Raw int32 accumulators of either grouped GEMM (inspection / parity only):
+ * acc[t, n] = sum_K a_q[t / row_div, K] * w[e_t, n, K] for every routed pair t.
+ * a_q int8 [*, K], w int8 [E, N, K] -> acc int32 [num_pairs, N].
+ */
+int moe_i8_gemm_acc_i32(const int8_t* a_q, const int8_t* w, const int32_t* sorted_token_ids,
+                        const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
+                        int64_t num_pairs, int row_div, int num_experts, int n, int k,
+                        int block_size, int64_t sorted_cap, int32_t* acc_out, int variant,
+                        void* stream);
+
+/*
+ * Replaces vLLM `ops.moe_sum(input, output)` (csrc/moe/moe_align_sum_kernels.cu);
+ * in-tree analogue: scatter_add combine, trainer/distributed/token_dispatcher.py:162-165.
+ * in bf16 [M, top_k, H] -> out bf16 [M, H].
+ */
+int moe_i8_sum(const void* in, void* out, int64_t m, int top_k, int hidden, void* stream);
+
+/* Bytes of caller-owned workspace moe_i8_fused_experts needs. */
+int64_t moe_i8_workspace_bytes(int64_t m, int top_k, int num_experts, int hidden, int inter,
+                               int block_size);
+
+/*
+ * Replaces vLLM `fused_experts(hidden_states, w1, w2, topk_weights, topk_ids,
+ * use_int8_w8a8=True, per_channel_quant=True, w1_scale, w2_scale,
+ * a1_scale=None, a2_scale=None)` -> `fused_experts_impl`
+ * (model_executor/layers/fused_moe/fused_moe.py): quant, align, gate_up GEMM +
+ * SiLU*mul, quant, down GEMM * routed weight, sum — all on `stream`, no host
+ * synchronisation.  hidden bf16 [M, H]; out bf16 [M, H] (may alias hidden).
+ */
+int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
+                         const float* topk_weights, const int32_t* topk_ids,
+                         const float* w1_scale, const float* w2_scale, void* out, int64_t m,
+                         int top_k, int num_experts, int hidden_size, int inter, int block_size,
+                         void* workspace, int64_t workspace_bytes, int variant, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE_I8_H_ */

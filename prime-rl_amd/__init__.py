@@ -1,0 +1,33 @@
+"""gfx950-native INT8 W8A8 fused-MoE path (drop-in for vLLM's ``fused_experts``).
+
+The directory name carries a hyphen, so import it through the top-level ``prime_rl_amd`` module
+(``import prime_rl_amd``), which aliases this package and its submodules.
+"""
+
+from . import _abi, inputs  # noqa: F401
+from .api import (  # noqa: F401
+    DEFAULT_BLOCK_SIZE_M,
+    fused_experts,
+    gemm_acc_i32,
+    gemm_down,
+    gemm_gate_up_silu,
+    moe_align_block_size,
+    moe_sum,
+    per_token_quant_int8,
+    sorted_capacity,
+    workspace_bytes,
+)
+from . import api, build, vllm_plugin  # noqa: F401
+
+__all__ = [
+    "fused_experts",
+    "moe_align_block_size",
+    "per_token_quant_int8",
+    "moe_sum",
+    "gemm_gate_up_silu",
+    "gemm_down",
+    "gemm_acc_i32",
+    "workspace_bytes",
+    "sorted_capacity",
+    "DEFAULT_BLOCK_SIZE_M",
+]

@@ -1,0 +1,370 @@
+"""Host side of the gfx950 INT8 W8A8 fused-MoE path, with vLLM's call signatures.
+
+``fused_experts`` keeps the flat signature of vLLM 0.28.0's
+``vllm.model_executor.layers.fused_moe.fused_experts`` (the function the reference's rollout
+engine reaches through the ``quantization`` pass-through,
+``packages/prime-rl-configs/src/prime_rl/configs/inference.py:108-109``), and
+``moe_align_block_size`` / ``per_token_quant_int8`` / ``moe_sum`` keep the names and returns of the
+pieces it is made of.  Everything runs in hand-written HIP kernels behind the C-ABI of
+``libmoe_i8.so``; torch only supplies device memory and the current stream.  There is no CPU or
+eager fallback: without the built library, or off a GPU, these functions raise.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _abi
+
+__all__ = [
+    "fused_experts",
+    "moe_align_block_size",
+    "per_token_quant_int8",
+    "moe_sum",
+    "gemm_gate_up_silu",
+    "gemm_down",
+    "gemm_acc_i32",
+    "workspace_bytes",
+    "sorted_capacity",
+    "DEFAULT_BLOCK_SIZE_M",
+]
+
+DEFAULT_BLOCK_SIZE_M = 64
+_VARIANTS = {"auto": _abi.GEMM_AUTO, "stream": _abi.GEMM_STREAM, "tile": _abi.GEMM_TILE}
+_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require_gpu(name: str, t: torch.Tensor) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a GPU tensor (this path has no CPU implementation)")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+
+
+def _variant(v: str | int) -> int:
+    if isinstance(v, int):
+        return v
+    try:
+        return _VARIANTS[v]
+    except KeyError:
+        raise ValueError(f"gemm variant must be one of {sorted(_VARIANTS)}") from None
+
+
+def _block_size(block_size: int) -> int:
+    if block_size not in (16, 32, 64, 128):
+        raise ValueError("block_size must be 16, 32, 64 or 128")
+    return int(block_size)
+
+
+def _as_i32_ids(topk_ids: torch.Tensor) -> torch.Tensor:
+    if topk_ids.dtype == torch.int32:
+        return topk_ids
+    if topk_ids.dtype in (torch.int64, torch.int16, torch.uint8):
+        return topk_ids.to(torch.int32)
+    raise ValueError(f"topk_ids must be an integer tensor, got {topk_ids.dtype}")
+
+
+def sorted_capacity(num_pairs: int, num_experts: int, block_size: int) -> int:
+    """Length of ``sorted_token_ids``: ``min(P + E*(B-1), P*B)`` as upstream sizes it."""
+    return int(_abi.load().moe_i8_sorted_capacity(num_pairs, num_experts, block_size))
+
+
+def workspace_bytes(m: int, top_k: int, num_experts: int, hidden: int, inter: int, block_size: int) -> int:
+    n = int(_abi.load().moe_i8_workspace_bytes(m, top_k, num_experts, hidden, inter, block_size))
+    if n < 0:
+        raise ValueError("invalid shape for workspace_bytes")
+    return n
+
+
+# --------------------------------------------------------------------------------------------- #
+def moe_align_block_size(
+    topk_ids: torch.Tensor,
+    block_size: int,
+    num_experts: int,
+    expert_map: torch.Tensor | None = None,
+    pad_sorted_ids: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """vLLM ``moe_align_block_size``: returns ``(sorted_token_ids, expert_ids, num_tokens_post_padded)``.
+
+    ``sorted_token_ids`` holds flat pair indices ``m*k + j`` grouped by expert in ascending order
+    (the reference's stable sort, ``trainer/distributed/token_dispatcher.py:145``), each expert
+    padded to a multiple of ``block_size`` with the sentinel ``topk_ids.numel()``; the unused tail
+    is all sentinel and unused ``expert_ids`` are ``-1``.
+    """
+    if expert_map is not None:
+        raise NotImplementedError("expert_map (expert parallelism) is not supported on this path")
+    _require_gpu("topk_ids", topk_ids)
+    block_size = _block_size(block_size)
+    if not 1 <= num_experts <= _abi.MAX_EXPERTS:
+        raise ValueError(f"num_experts must be in [1, {_abi.MAX_EXPERTS}]")
+    lib = _abi.load()
+    ids = _as_i32_ids(topk_ids)
+    P = ids.numel()
+    cap = sorted_capacity(P, num_experts, block_size)
+    if pad_sorted_ids:
+        cap = (cap + block_size - 1) // block_size * block_size
+    dev = ids.device
+    sorted_ids = torch.empty((cap,), dtype=torch.int32, device=dev)
+    expert_ids = torch.empty(((cap + block_size - 1) // block_size,), dtype=torch.int32, device=dev)
+    npp = torch.empty((1,), dtype=torch.int32, device=dev)
+    ws_bytes = int(lib.moe_i8_align_workspace_bytes(P, num_experts, block_size))
+    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+    _abi.check(
+        lib.moe_i8_align_block_size(
+            _ptr(ids), P, num_experts, block_size, _ptr(sorted_ids), cap, _ptr(expert_ids),
+            expert_ids.numel(), _ptr(npp), _ptr(ws), ws_bytes, _stream(ids),
+        )
+    )
+    return sorted_ids, expert_ids, npp
+
+
+def per_token_quant_int8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """vLLM ``per_token_quant_int8``: ``(x_q int8 like x, scales fp32 [..., 1])``, fp32 arithmetic,
+    ``scale = max(absmax, 1e-10) / 127``, rounding half away from zero."""
+    _require_gpu("x", x)
+    if x.dtype != torch.bfloat16:
+        raise NotImplementedError(f"only bfloat16 activations are supported, got {x.dtype}")
+    cols = x.shape[-1]
+    if cols % 8 or cols == 0:
+        raise ValueError("last dimension must be a positive multiple of 8")
+    rows = x.numel() // cols
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    scale = torch.empty((*x.shape[:-1], 1), dtype=torch.float32, device=x.device)
+    _abi.check(
+        _abi.load().moe_i8_quant_rows(
+            _ptr(x), _abi.DTYPE_BF16, rows, cols, cols, None, 1, rows, _ptr(q), _ptr(scale), _stream(x)
+        )
+    )
+    return q, scale
+
+
+def moe_sum(input: torch.Tensor, output: torch.Tensor) -> None:
+    """vLLM ``ops.moe_sum``: ``output[m] = sum_j input[m, j]`` for bf16 ``[M, k, H]`` → ``[M, H]``."""
+    _require_gpu("input", input)
+    _require_gpu("output", output)
+    if input.dtype != torch.bfloat16 or output.dtype != torch.bfloat16:
+        raise NotImplementedError("only bfloat16 is supported")
+    if input.dim() != 3 or output.shape != (input.shape[0], input.shape[2]):
+        raise ValueError("expected input [M, k, H] and output [M, H]")
+    M, k, H = input.shape
+    if H % 8:
+        raise ValueError("hidden size must be a multiple of 8")
+    _abi.check(_abi.load().moe_i8_sum(_ptr(input), _ptr(output), M, k, H, _stream(input)))
+
+
+# --------------------------------------------------------------------------------------------- #
+def _check_routing(sorted_token_ids, expert_ids, num_tokens_post_padded):
+    for name, t in (
+        ("sorted_token_ids", sorted_token_ids),
+        ("expert_ids", expert_ids),
+        ("num_tokens_post_padded", num_tokens_post_padded),
+    ):
+        _require_gpu(name, t)
+        if t.dtype != torch.int32:
+            raise ValueError(f"{name} must be int32")
+
+
+def _check_weights(name: str, w: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    _require_gpu(name, w)
+    if w.dtype != torch.int8 or w.dim() != 3:
+        raise ValueError(f"{name} must be int8 [E, N, K]")
+    _require_gpu(name + "_scale", scale)
+    if scale.dtype != torch.float32:
+        raise ValueError(f"{name}_scale must be float32")
+    E, N, _ = w.shape
+    if scale.numel() != E * N:
+        raise NotImplementedError(f"{name}_scale must be per output channel, [E, N] or [E, N, 1]")
+    return scale.reshape(E, N)
+
+
+def gemm_gate_up_silu(
+    x_q, a_scale, w1, w1_scale, sorted_token_ids, expert_ids, num_tokens_post_padded,
+    top_k: int, block_size: int, num_pairs: int, variant: str | int = "auto",
+) -> torch.Tensor:
+    """Grouped gate_up GEMM on int8 MFMA with scale epilogue and fused SiLU·mul → bf16 ``[P, I]``."""
+    _require_gpu("x_q", x_q)
+    _check_routing(sorted_token_ids, expert_ids, num_tokens_post_padded)
+    w1_scale = _check_weights("w1", w1, w1_scale)
+    E, N, H = w1.shape
+    if x_q.dtype != torch.int8 or x_q.dim() != 2 or x_q.shape[1] != H:
+        raise ValueError("x_q must be int8 [M, H]")
+    if N % 2:
+        raise ValueError("w1 must stack gate and up: [E, 2I, H]")
+    a_scale = a_scale.reshape(-1)
+    out = torch.empty((num_pairs, N // 2), dtype=torch.bfloat16, device=x_q.device)
+    _abi.check(
+        _abi.load().moe_i8_gemm_gate_up_silu(
+            _ptr(x_q), _ptr(a_scale), _ptr(w1), _ptr(w1_scale), _ptr(sorted_token_ids),
+            _ptr(expert_ids), _ptr(num_tokens_post_padded), num_pairs, top_k, E, H, N // 2,
+            _block_size(block_size), sorted_token_ids.numel(), _ptr(out), _variant(variant),
+            _stream(x_q),
+        )
+    )
+    return out
+
+
+def gemm_down(
+    h_q, a_scale, w2, w2_scale, topk_weights, sorted_token_ids, expert_ids,
+    num_tokens_post_padded, block_size: int, variant: str | int = "auto",
+) -> torch.Tensor:
+    """Grouped down GEMM on int8 MFMA, scales and routed weight in the epilogue → bf16 ``[P, H]``."""
+    _require_gpu("h_q", h_q)
+    _check_routing(sorted_token_ids, expert_ids, num_tokens_post_padded)
+    w2_scale = _check_weights("w2", w2, w2_scale)
+    E, H, I = w2.shape
+    if h_q.dtype != torch.int8 or h_q.dim() != 2 or h_q.shape[1] != I:
+        raise ValueError("h_q must be int8 [P, I]")
+    P = h_q.shape[0]
+    tw = topk_weights.reshape(-1)
+    if tw.dtype != torch.float32 or tw.numel() != P:
+        raise ValueError("topk_weights must be float32 with one entry per pair")
+    a_scale = a_scale.reshape(-1)
+    out = torch.empty((P, H), dtype=torch.bfloat16, device=h_q.device)
+    _abi.check(
+        _abi.load().moe_i8_gemm_down(
+            _ptr(h_q), _ptr(a_scale), _ptr(w2), _ptr(w2_scale), _ptr(tw), _ptr(sorted_token_ids),
+            _ptr(expert_ids), _ptr(num_tokens_post_padded), P, E, H, I, _block_size(block_size),
+            sorted_token_ids.numel(), _ptr(out), _variant(variant), _stream(h_q),
+        )
+    )
+    return out
+
+
+def gemm_acc_i32(
+    a_q, w, sorted_token_ids, expert_ids, num_tokens_post_padded, row_div: int, block_size: int,
+    num_pairs: int, variant: str | int = "auto",
+) -> torch.Tensor:
+    """Raw int32 accumulators ``acc[t, n] = Σ_K a_q[t // row_div, K]·w[e_t, n, K]`` → int32 ``[P, N]``
+    (rows of pairs whose expert id is out of range are left zero)."""
+    _require_gpu("a_q", a_q)
+    _require_gpu("w", w)
+    _check_routing(sorted_token_ids, expert_ids, num_tokens_post_padded)
+    E, N, K = w.shape
+    if a_q.dtype != torch.int8 or w.dtype != torch.int8 or a_q.shape[-1] != K:
+        raise ValueError("a_q int8 [*, K] and w int8 [E, N, K] expected")
+    out = torch.zeros((num_pairs, N), dtype=torch.int32, device=a_q.device)
+    _abi.check(
+        _abi.load().moe_i8_gemm_acc_i32(
+            _ptr(a_q), _ptr(w), _ptr(sorted_token_ids), _ptr(expert_ids),
+            _ptr(num_tokens_post_padded), num_pairs, row_div, E, N, K, _block_size(block_size),
+            sorted_token_ids.numel(), _ptr(out), _variant(variant), _stream(a_q),
+        )
+    )
+    return out
+
+
+# --------------------------------------------------------------------------------------------- #
+def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def fused_experts(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    topk_weights: torch.Tensor,
+    topk_ids: torch.Tensor,
+    inplace: bool = False,
+    activation: str = "silu",
+    apply_router_weight_on_input: bool = False,
+    use_int8_w8a8: bool = False,
+    per_channel_quant: bool = False,
+    global_num_experts: int = -1,
+    expert_map: torch.Tensor | None = None,
+    w1_scale: torch.Tensor | None = None,
+    w2_scale: torch.Tensor | None = None,
+    a1_scale: torch.Tensor | None = None,
+    a2_scale: torch.Tensor | None = None,
+    block_shape: list[int] | None = None,
+    *,
+    block_size_m: int = DEFAULT_BLOCK_SIZE_M,
+    gemm_variant: str | int = "auto",
+    workspace: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Drop-in for vLLM ``fused_experts`` on the INT8 W8A8 path (per-channel weight scales, dynamic
+    per-token activation scales, SiLU-gated experts, routed weight applied after the experts).
+
+    ``a1_scale`` / ``a2_scale`` are accepted for signature compatibility and ignored: with
+    per-token dynamic quantisation upstream recomputes them too.  The three keyword-only
+    arguments are extensions: the moe_align block size (64, as the baseline pins it), the GEMM
+    kernel family and an optional caller-owned workspace of ``workspace_bytes(...)`` bytes.
+    """
+    if not use_int8_w8a8:
+        raise NotImplementedError("this library implements only the use_int8_w8a8=True path")
+    if not per_channel_quant:
+        raise NotImplementedError("int8 W8A8 MoE requires per_channel_quant=True (channel-wise weights)")
+    if activation != "silu":
+        raise NotImplementedError(f"activation {activation!r} is not supported (only 'silu')")
+    if apply_router_weight_on_input:
+        raise NotImplementedError("apply_router_weight_on_input=True is not supported")
+    if expert_map is not None:
+        raise NotImplementedError("expert_map (expert parallelism) is not supported on this path")
+    if block_shape is not None:
+        raise NotImplementedError("block-wise quantisation (block_shape) is not supported")
+    if w1_scale is None or w2_scale is None:
+        raise ValueError("w1_scale and w2_scale are required for use_int8_w8a8")
+    _require_gpu("hidden_states", hidden_states)
+    if hidden_states.dtype != torch.bfloat16:
+        raise NotImplementedError(f"only bfloat16 hidden_states are supported, got {hidden_states.dtype}")
+    if hidden_states.dim() != 2:
+        raise ValueError("hidden_states must be [M, H]")
+    w1_scale = _check_weights("w1", w1, w1_scale)
+    w2_scale = _check_weights("w2", w2, w2_scale)
+    M, H = hidden_states.shape
+    E, N1, K1 = w1.shape
+    if K1 != H:
+        raise ValueError(f"hidden size mismatch: hidden_states {H} vs w1 {K1}")
+    if N1 % 2:
+        raise ValueError("w1 must stack gate and up: [E, 2I, H]")
+    I = N1 // 2
+    if tuple(w2.shape) != (E, H, I):
+        raise ValueError(f"w2 must be [E, H, I] = {(E, H, I)}, got {tuple(w2.shape)}")
+    if global_num_experts not in (-1, E):
+        raise NotImplementedError("global_num_experts != local expert count needs expert_map")
+    if E > _abi.MAX_EXPERTS:
+        raise ValueError(f"at most {_abi.MAX_EXPERTS} experts are supported")
+    if H % 64 or I % 64:
+        raise ValueError("hidden and intermediate sizes must be multiples of 64")
+    if topk_weights.shape != topk_ids.shape or topk_ids.dim() != 2 or topk_ids.shape[0] != M:
+        raise ValueError("topk_weights and topk_ids must both be [M, k]")
+    _require_gpu("topk_ids", topk_ids)
+    _require_gpu("topk_weights", topk_weights)
+    block_size_m = _block_size(block_size_m)
+    k = topk_ids.shape[1]
+    out = hidden_states if inplace else torch.empty_like(hidden_states)
+    if M == 0:
+        return out
+    ids = _as_i32_ids(topk_ids)
+    tw = topk_weights if topk_weights.dtype == torch.float32 else topk_weights.to(torch.float32)
+    lib = _abi.load()
+    need = workspace_bytes(M, k, E, H, I, block_size_m)
+    stream = _stream(hidden_states)
+    if workspace is None:
+        workspace = _workspace(hidden_states.device, stream, need)
+    else:
+        _require_gpu("workspace", workspace)
+        if workspace.numel() * workspace.element_size() < need:
+            raise ValueError(f"workspace too small: need {need} bytes")
+    _abi.check(
+        lib.moe_i8_fused_experts(
+            _ptr(hidden_states), _ptr(w1), _ptr(w2), _ptr(tw), _ptr(ids), _ptr(w1_scale),
+            _ptr(w2_scale), _ptr(out), M, k, E, H, I, block_size_m, _ptr(workspace),
+            workspace.numel() * workspace.element_size(), _variant(gemm_variant), stream,
+        )
+    )
+    return out

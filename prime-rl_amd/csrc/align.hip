@@ -1,0 +1,291 @@
+// moe_align_block_size for gfx950: stable counting sort of (token, expert) pairs by expert,
+// each expert segment padded to a multiple of the block size.
+//
+// The unit of work is one 64-lane wavefront walking a contiguous chunk of pairs.  Inside a
+// wavefront the rank of a pair among the lanes that hold the same expert comes from ballots
+// (one per bit of the expert id) and a population count below the lane, so no atomics are
+// needed and the order inside an expert segment is the ascending flat pair index.
+//
+// Small inputs run in one 1024-thread workgroup (histogram, scans and scatter fused).  Large
+// inputs use three launches: per-wave histograms, one scan workgroup, scatter.
+#include "common.hpp"
+
+namespace moe_i8 {
+namespace {
+
+constexpr int kSingleThreads = 1024;
+constexpr int kSingleWaves = kSingleThreads / kWave;
+constexpr int kMultiThreads = 256;
+constexpr int kMultiWaves = kMultiThreads / kWave;
+constexpr int kMultiChunk = 1024;         // pairs per wavefront in the multi-launch path
+constexpr int64_t kSingleMaxPairs = 8192;  // above this the multi-launch path is used
+
+// Lanes of this wavefront that are active and hold the same expert id as the caller.
+__device__ __forceinline__ uint64_t peers_of(int e, bool active, int nbits) {
+  uint64_t m = __ballot(active);
+  for (int b = 0; b < nbits; ++b) {
+    const bool bit = (e >> b) & 1;
+    const uint64_t bm = __ballot(active && bit);
+    m &= bit ? bm : ~bm;
+  }
+  return m;
+}
+
+// counts[e] += number of pairs in [begin, end) routed to e; counts is private to the wavefront.
+__device__ __forceinline__ void wave_histogram(const int32_t* __restrict__ ids, int64_t begin,
+                                               int64_t end, int E, int nbits, int* counts) {
+  const int lane = lane_id();
+  for (int64_t base = begin; base < end; base += kWave) {
+    const int64_t idx = base + lane;
+    int e = idx < end ? ids[idx] : -1;
+    const bool active = e >= 0 && e < E;
+    const uint64_t peers = peers_of(e, active, nbits);
+    const int rank = __popcll(peers & ((1ull << lane) - 1ull));
+    if (active && rank == 0) counts[e] += __popcll(peers);
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// sorted[cursor[e]++] = idx for the pairs in [begin, end), in ascending idx order per expert.
+__device__ __forceinline__ void wave_scatter(const int32_t* __restrict__ ids, int64_t begin,
+                                             int64_t end, int E, int nbits, int* cursor,
+                                             int32_t* __restrict__ sorted, int64_t sorted_cap) {
+  const int lane = lane_id();
+  for (int64_t base = begin; base < end; base += kWave) {
+    const int64_t idx = base + lane;
+    int e = idx < end ? ids[idx] : -1;
+    const bool active = e >= 0 && e < E;
+    const uint64_t peers = peers_of(e, active, nbits);
+    const int rank = __popcll(peers & ((1ull << lane) - 1ull));
+    int pos = 0;
+    if (active) pos = cursor[e] + rank;
+    __builtin_amdgcn_wave_barrier();
+    if (active && rank == 0) cursor[e] += __popcll(peers);
+    __builtin_amdgcn_wave_barrier();
+    if (active && pos < sorted_cap) sorted[pos] = (int32_t)idx;
+  }
+}
+
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+  const int lane = lane_id();
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int n = __shfl_up(v, d);
+    if (lane >= d) v += n;
+  }
+  return v;
+}
+
+// Exclusive scan over the 1024 threads of the block; returns the exclusive prefix, *total = sum.
+__device__ __forceinline__ int block_exclusive_scan_1024(int v, int* wave_sums, int* total) {
+  const int lane = lane_id();
+  const int wave = threadIdx.x / kWave;
+  const int incl = wave_inclusive_scan(v);
+  if (lane == kWave - 1) wave_sums[wave] = incl;
+  __syncthreads();
+  if (wave == 0) {
+    const int s = lane < kSingleWaves ? wave_sums[lane] : 0;
+    const int si = wave_inclusive_scan(s);
+    if (lane < kSingleWaves) wave_sums[lane] = si - s;
+    if (lane == kSingleWaves - 1) wave_sums[kSingleWaves] = si;
+  }
+  __syncthreads();
+  *total = wave_sums[kSingleWaves];
+  return wave_sums[wave] + incl - v;
+}
+
+// From per-expert padded segment starts (seg[0..E], seg[E] = total) write expert_ids.
+__device__ __forceinline__ void write_expert_ids(const int* seg, int E, int B, int npp,
+                                                 int32_t* __restrict__ expert_ids,
+                                                 int64_t expert_cap) {
+  for (int64_t j = threadIdx.x; j < expert_cap; j += blockDim.x) {
+    const int64_t pos = j * B;
+    int e = -1;
+    if (pos < npp) {
+      // largest e with seg[e] <= pos (an empty expert shares its start with its successor)
+      int lo = 0, hi = E - 1;
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (seg[mid] <= pos) lo = mid; else hi = mid - 1;
+      }
+      e = lo;
+    }
+    expert_ids[j] = e;
+  }
+}
+
+// LDS layout: hist[kSingleWaves][E] | seg[E + 1] | wave_sums[kSingleWaves + 1]
+__global__ __launch_bounds__(kSingleThreads) void align_single_kernel(
+    const int32_t* __restrict__ ids, int P, int E, int B, int nbits,
+    int32_t* __restrict__ sorted, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
+    int64_t expert_cap, int32_t* __restrict__ npp_out) {
+  extern __shared__ int smem[];
+  int* hist = smem;
+  int* seg = hist + kSingleWaves * E;
+  int* wave_sums = seg + E + 1;
+  const int tid = threadIdx.x;
+  const int wave = tid / kWave;
+
+  for (int i = tid; i < kSingleWaves * E; i += kSingleThreads) hist[i] = 0;
+  for (int64_t i = tid; i < sorted_cap; i += kSingleThreads) sorted[i] = P;
+  __syncthreads();
+
+  const int per_wave = ((P + kSingleWaves - 1) / kSingleWaves + kWave - 1) / kWave * kWave;
+  const int64_t begin = (int64_t)wave * per_wave < P ? (int64_t)wave * per_wave : P;
+  const int64_t end = begin + per_wave < P ? begin + per_wave : P;
+  wave_histogram(ids, begin, end, E, nbits, hist + wave * E);
+  __syncthreads();
+
+  int padded = 0;
+  if (tid < E) {
+    int run = 0;
+    for (int w = 0; w < kSingleWaves; ++w) {
+      const int c = hist[w * E + tid];
+      hist[w * E + tid] = run;
+      run += c;
+    }
+    padded = (run + B - 1) / B * B;
+  }
+  int npp;
+  const int start = block_exclusive_scan_1024(padded, wave_sums, &npp);
+  if (tid < E) seg[tid] = start;
+  if (tid == 0) {
+    seg[E] = npp;
+    *npp_out = npp;
+  }
+  __syncthreads();
+  if (tid < E)
+    for (int w = 0; w < kSingleWaves; ++w) hist[w * E + tid] += start;
+  write_expert_ids(seg, E, B, npp, expert_ids, expert_cap);
+  __syncthreads();
+  wave_scatter(ids, begin, end, E, nbits, hist + wave * E, sorted, sorted_cap);
+}
+
+// ---- multi-launch path -------------------------------------------------------------------
+// workspace: unit_hist[units][E] | seg[E + 1]
+
+__global__ __launch_bounds__(kMultiThreads) void align_hist_kernel(
+    const int32_t* __restrict__ ids, int64_t P, int E, int nbits, int units,
+    int32_t* __restrict__ unit_hist, int32_t* __restrict__ sorted, int64_t sorted_cap) {
+  extern __shared__ int smem[];
+  const int tid = threadIdx.x;
+  const int wave = tid / kWave;
+  for (int64_t i = (int64_t)blockIdx.x * kMultiThreads + tid; i < sorted_cap;
+       i += (int64_t)gridDim.x * kMultiThreads)
+    sorted[i] = (int32_t)P;
+  for (int i = tid; i < kMultiWaves * E; i += kMultiThreads) smem[i] = 0;
+  __syncthreads();
+  const int unit = blockIdx.x * kMultiWaves + wave;
+  if (unit < units) {
+    const int64_t begin = (int64_t)unit * kMultiChunk;
+    const int64_t end = begin + kMultiChunk < P ? begin + kMultiChunk : P;
+    wave_histogram(ids, begin, end, E, nbits, smem + wave * E);
+  }
+  __syncthreads();
+  for (int i = tid; i < kMultiWaves * E; i += kMultiThreads) {
+    const int u = blockIdx.x * kMultiWaves + i / E;
+    if (u < units) unit_hist[(int64_t)u * E + i % E] = smem[i];
+  }
+}
+
+__global__ __launch_bounds__(kSingleThreads) void align_scan_kernel(
+    int E, int B, int units, int32_t* __restrict__ unit_hist, int32_t* __restrict__ seg_out,
+    int32_t* __restrict__ expert_ids, int64_t expert_cap, int32_t* __restrict__ npp_out) {
+  __shared__ int seg[kMaxExperts + 1];
+  __shared__ int wave_sums[kSingleWaves + 1];
+  const int tid = threadIdx.x;
+  int padded = 0;
+  if (tid < E) {
+    int run = 0;
+#pragma unroll 8
+    for (int u = 0; u < units; ++u) {
+      const int c = unit_hist[(int64_t)u * E + tid];
+      unit_hist[(int64_t)u * E + tid] = run;
+      run += c;
+    }
+    padded = (run + B - 1) / B * B;
+  }
+  int npp;
+  const int start = block_exclusive_scan_1024(padded, wave_sums, &npp);
+  if (tid < E) {
+    seg[tid] = start;
+    seg_out[tid] = start;
+  }
+  if (tid == 0) {
+    seg[E] = npp;
+    seg_out[E] = npp;
+    *npp_out = npp;
+  }
+  __syncthreads();
+  write_expert_ids(seg, E, B, npp, expert_ids, expert_cap);
+}
+
+__global__ __launch_bounds__(kMultiThreads) void align_scatter_kernel(
+    const int32_t* __restrict__ ids, int64_t P, int E, int nbits, int units,
+    const int32_t* __restrict__ unit_hist, const int32_t* __restrict__ seg,
+    int32_t* __restrict__ sorted, int64_t sorted_cap) {
+  extern __shared__ int smem[];
+  const int tid = threadIdx.x;
+  const int wave = tid / kWave;
+  for (int i = tid; i < kMultiWaves * E; i += kMultiThreads) {
+    const int u = blockIdx.x * kMultiWaves + i / E;
+    const int e = i % E;
+    smem[i] = u < units ? seg[e] + unit_hist[(int64_t)u * E + e] : 0;
+  }
+  __syncthreads();
+  const int unit = blockIdx.x * kMultiWaves + wave;
+  if (unit < units) {
+    const int64_t begin = (int64_t)unit * kMultiChunk;
+    const int64_t end = begin + kMultiChunk < P ? begin + kMultiChunk : P;
+    wave_scatter(ids, begin, end, E, nbits, smem + wave * E, sorted, sorted_cap);
+  }
+}
+
+int bits_for(int E) {
+  int b = 0;
+  while ((1 << b) < E) ++b;
+  return b;
+}
+
+}  // namespace
+
+int64_t align_workspace_ints(int64_t num_pairs, int num_experts) {
+  if (num_pairs <= kSingleMaxPairs) return 0;
+  const int64_t units = (num_pairs + kMultiChunk - 1) / kMultiChunk;
+  return units * num_experts + num_experts + 1;
+}
+
+hipError_t launch_align(const AlignArgs& a, hipStream_t stream) {
+  const int E = a.num_experts;
+  const int nbits = bits_for(E);
+  if (a.num_pairs <= kSingleMaxPairs) {
+    const size_t lds = sizeof(int) * ((size_t)kSingleWaves * E + E + 1 + kSingleWaves + 1);
+    static const hipError_t attr = hipFuncSetAttribute(
+        (const void*)align_single_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+        (int)(sizeof(int) * ((size_t)kSingleWaves * kMaxExperts + kMaxExperts + kSingleWaves + 2)));
+    if (attr != hipSuccess) return attr;
+    hipLaunchKernelGGL(align_single_kernel, dim3(1), dim3(kSingleThreads), lds, stream, a.topk_ids,
+                       (int)a.num_pairs, E, a.block_size, nbits, a.sorted_token_ids, a.sorted_cap,
+                       a.expert_ids, a.expert_cap, a.num_tokens_post_padded);
+    return hipGetLastError();
+  }
+  const int units = (int)((a.num_pairs + kMultiChunk - 1) / kMultiChunk);
+  const int blocks = (units + kMultiWaves - 1) / kMultiWaves;
+  int32_t* unit_hist = a.workspace;
+  int32_t* seg = a.workspace + (int64_t)units * E;
+  const size_t lds = sizeof(int) * (size_t)kMultiWaves * E;
+  hipLaunchKernelGGL(align_hist_kernel, dim3(blocks), dim3(kMultiThreads), lds, stream, a.topk_ids,
+                     a.num_pairs, E, nbits, units, unit_hist, a.sorted_token_ids, a.sorted_cap);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kSingleThreads), 0, stream, E, a.block_size,
+                     units, unit_hist, seg, a.expert_ids, a.expert_cap, a.num_tokens_post_padded);
+  err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  hipLaunchKernelGGL(align_scatter_kernel, dim3(blocks), dim3(kMultiThreads), lds, stream,
+                     a.topk_ids, a.num_pairs, E, nbits, units, unit_hist, seg, a.sorted_token_ids,
+                     a.sorted_cap);
+  return hipGetLastError();
+}
+
+}  // namespace moe_i8

@@ -1,0 +1,351 @@
+// C-ABI of libmoe_i8.so: argument validation, workspace carving and kernel launches.
+// Nothing here allocates device memory or synchronises; every launch goes to the caller's stream.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/moe_i8.h"
+#include "common.hpp"
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(hipError_t err, const char* what) {
+  if (err == hipSuccess) return MOE_I8_OK;
+  return fail(MOE_I8_ELAUNCH, "%s: %s", what, hipGetErrorString(err));
+}
+
+bool valid_block_size(int b) { return b == 16 || b == 32 || b == 64 || b == 128; }
+
+int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_gemm_common(const void* a_q, const void* w, const int32_t* sorted, const int32_t* eids,
+                      const int32_t* npp, const void* out, int64_t num_pairs, int num_experts,
+                      int n, int k, int block_size, int64_t sorted_cap, int variant) {
+  if (!a_q || !w || !sorted || !eids || !npp || !out) return fail(MOE_I8_EINVAL, "null pointer");
+  if (!aligned16(a_q) || !aligned16(w) || !aligned16(out))
+    return fail(MOE_I8_EINVAL, "activation, weight and output pointers must be 16-byte aligned");
+  if (num_pairs < 0 || num_pairs > INT32_MAX - 1) return fail(MOE_I8_EINVAL, "num_pairs out of range");
+  if (num_experts < 1 || num_experts > MOE_I8_MAX_EXPERTS)
+    return fail(MOE_I8_EINVAL, "num_experts must be in [1, %d]", MOE_I8_MAX_EXPERTS);
+  if (!valid_block_size(block_size)) return fail(MOE_I8_EINVAL, "block_size must be 16, 32, 64 or 128");
+  if (n < 16 || n % 16) return fail(MOE_I8_EINVAL, "output channels (%d) must be a positive multiple of 16", n);
+  if (k < 64 || k % 64) return fail(MOE_I8_EINVAL, "reduction length (%d) must be a positive multiple of 64", k);
+  if (sorted_cap < moe_i8_sorted_capacity(num_pairs, num_experts, block_size))
+    return fail(MOE_I8_EWORKSPACE, "sorted_token_ids capacity %lld too small", (long long)sorted_cap);
+  if (variant != MOE_I8_GEMM_AUTO && variant != MOE_I8_GEMM_STREAM && variant != MOE_I8_GEMM_TILE)
+    return fail(MOE_I8_EINVAL, "unknown GEMM variant %d", variant);
+  return MOE_I8_OK;
+}
+
+int run_gemm(const moe_i8::GemmArgs& g, int variant, hipStream_t stream) {
+  if (g.num_pairs == 0) return MOE_I8_OK;
+  bool tile;
+  if (variant == MOE_I8_GEMM_TILE) {
+    if (!moe_i8::gemm_tile_supports(g))
+      return fail(MOE_I8_EUNSUPPORTED, "tile GEMM does not support this shape");
+    tile = true;
+  } else if (variant == MOE_I8_GEMM_STREAM) {
+    tile = false;
+  } else {
+    // More than ~16 routed rows per expert on average: weights are reused enough for LDS tiles.
+    tile = moe_i8::gemm_tile_supports(g) && g.num_pairs > (int64_t)16 * g.num_experts;
+  }
+  return check_launch(tile ? moe_i8::launch_gemm_tile(g, stream) : moe_i8::launch_gemm_stream(g, stream),
+                      tile ? "gemm_tile" : "gemm_stream");
+}
+
+}  // namespace
+
+extern "C" {
+
+int moe_i8_version(void) { return 1; }
+
+const char* moe_i8_last_error(void) { return g_error; }
+
+int64_t moe_i8_sorted_capacity(int64_t num_pairs, int num_experts, int block_size) {
+  if (num_pairs < 0 || num_experts < 1 || block_size < 1) return -1;
+  const int64_t full = num_pairs + (int64_t)num_experts * (block_size - 1);
+  const int64_t tight = num_pairs * block_size;
+  return full < tight ? full : tight;
+}
+
+int64_t moe_i8_align_workspace_bytes(int64_t num_pairs, int num_experts, int block_size) {
+  (void)block_size;
+  if (num_pairs < 0 || num_experts < 1) return -1;
+  return moe_i8::align_workspace_ints(num_pairs, num_experts) * (int64_t)sizeof(int32_t);
+}
+
+int moe_i8_align_block_size(const int32_t* topk_ids, int64_t num_pairs, int num_experts,
+                            int block_size, int32_t* sorted_token_ids, int64_t sorted_cap,
+                            int32_t* expert_ids, int64_t expert_cap,
+                            int32_t* num_tokens_post_padded, void* workspace,
+                            int64_t workspace_bytes, void* stream) {
+  if (num_pairs < 0 || num_pairs > INT32_MAX - 1) return fail(MOE_I8_EINVAL, "num_pairs out of range");
+  if (num_experts < 1 || num_experts > MOE_I8_MAX_EXPERTS)
+    return fail(MOE_I8_EINVAL, "num_experts must be in [1, %d]", MOE_I8_MAX_EXPERTS);
+  if (!valid_block_size(block_size)) return fail(MOE_I8_EINVAL, "block_size must be 16, 32, 64 or 128");
+  if (!num_tokens_post_padded || (num_pairs > 0 && !topk_ids))
+    return fail(MOE_I8_EINVAL, "null pointer");
+  const int64_t need = moe_i8_sorted_capacity(num_pairs, num_experts, block_size);
+  if (sorted_cap < need)
+    return fail(MOE_I8_EWORKSPACE, "sorted_token_ids capacity %lld < %lld", (long long)sorted_cap,
+                (long long)need);
+  if (expert_cap < (sorted_cap + block_size - 1) / block_size)
+    return fail(MOE_I8_EWORKSPACE, "expert_ids capacity %lld too small", (long long)expert_cap);
+  if ((sorted_cap > 0 && !sorted_token_ids) || (expert_cap > 0 && !expert_ids))
+    return fail(MOE_I8_EINVAL, "null pointer");
+  const int64_t ws_need = moe_i8_align_workspace_bytes(num_pairs, num_experts, block_size);
+  if (ws_need > 0 && (!workspace || workspace_bytes < ws_need))
+    return fail(MOE_I8_EWORKSPACE, "align workspace %lld < %lld bytes", (long long)workspace_bytes,
+                (long long)ws_need);
+  moe_i8::AlignArgs a;
+  a.topk_ids = topk_ids;
+  a.num_pairs = num_pairs;
+  a.num_experts = num_experts;
+  a.block_size = block_size;
+  a.sorted_token_ids = sorted_token_ids;
+  a.sorted_cap = sorted_cap;
+  a.expert_ids = expert_ids;
+  a.expert_cap = expert_cap;
+  a.num_tokens_post_padded = num_tokens_post_padded;
+  a.workspace = static_cast<int32_t*>(workspace);
+  return check_launch(moe_i8::launch_align(a, static_cast<hipStream_t>(stream)), "moe_align");
+}
+
+int moe_i8_quant_rows(const void* x, int dtype, int64_t src_rows, int64_t cols, int64_t row_stride,
+                      const int32_t* gather, int gather_div, int64_t rows, int8_t* q, float* scale,
+                      void* stream) {
+  if (dtype != MOE_I8_DTYPE_BF16) return fail(MOE_I8_EUNSUPPORTED, "only bf16 activations are supported");
+  if (rows < 0 || src_rows < 0) return fail(MOE_I8_EINVAL, "negative row count");
+  if (rows == 0) return MOE_I8_OK;
+  if (!x || !q || !scale) return fail(MOE_I8_EINVAL, "null pointer");
+  if (cols < 8 || cols % 8 || cols > INT32_MAX) return fail(MOE_I8_EINVAL, "cols (%lld) must be a positive multiple of 8", (long long)cols);
+  if (row_stride < cols || row_stride % 8) return fail(MOE_I8_EINVAL, "row stride must be >= cols and a multiple of 8");
+  if (!aligned16(x) || (reinterpret_cast<uintptr_t>(q) & 7u))
+    return fail(MOE_I8_EINVAL, "x must be 16-byte and q 8-byte aligned");
+  if (gather && gather_div < 1) return fail(MOE_I8_EINVAL, "gather_div must be >= 1");
+  if (!gather && rows > src_rows) return fail(MOE_I8_EINVAL, "rows exceeds src_rows");
+  moe_i8::QuantArgs a;
+  a.x = static_cast<const uint16_t*>(x);
+  a.src_rows = src_rows;
+  a.cols = (int)cols;
+  a.row_stride = row_stride;
+  a.gather = gather;
+  a.gather_div = gather ? gather_div : 1;
+  a.rows = rows;
+  a.q = q;
+  a.scale = scale;
+  return check_launch(moe_i8::launch_quant_rows(a, static_cast<hipStream_t>(stream)), "quant_rows");
+}
+
+int moe_i8_gemm_gate_up_silu(const int8_t* x_q, const float* a_scale, const int8_t* w1,
+                             const float* w1_scale, const int32_t* sorted_token_ids,
+                             const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
+                             int64_t num_pairs, int top_k, int num_experts, int hidden, int inter,
+                             int block_size, int64_t sorted_cap, void* act_out, int variant,
+                             void* stream) {
+  if (num_pairs == 0) return MOE_I8_OK;
+  if (inter < 16 || inter % 16 || inter > (1 << 29)) return fail(MOE_I8_EINVAL, "inter (%d) must be a positive multiple of 16", inter);
+  if (int rc = check_gemm_common(x_q, w1, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                                 act_out, num_pairs, num_experts, 2 * inter, hidden, block_size,
+                                 sorted_cap, variant))
+    return rc;
+  if (!a_scale || !w1_scale) return fail(MOE_I8_EINVAL, "null scale pointer");
+  if (!aligned16(w1_scale)) return fail(MOE_I8_EINVAL, "w1_scale must be 16-byte aligned");
+  if (top_k < 1) return fail(MOE_I8_EINVAL, "top_k must be >= 1");
+  moe_i8::GemmArgs g{};
+  g.mode = moe_i8::kGateUpSilu;
+  g.a_q = x_q;
+  g.a_scale = a_scale;
+  g.w = w1;
+  g.w_scale = w1_scale;
+  g.row_weight = nullptr;
+  g.sorted_token_ids = sorted_token_ids;
+  g.expert_ids = expert_ids;
+  g.num_tokens_post_padded = num_tokens_post_padded;
+  g.num_pairs = num_pairs;
+  g.row_div = top_k;
+  g.num_experts = num_experts;
+  g.n = 2 * inter;
+  g.k = hidden;
+  g.block_size = block_size;
+  g.sorted_cap = sorted_cap;
+  g.out = act_out;
+  return run_gemm(g, variant, static_cast<hipStream_t>(stream));
+}
+
+int moe_i8_gemm_down(const int8_t* h_q, const float* a_scale, const int8_t* w2,
+                     const float* w2_scale, const float* topk_weights,
+                     const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                     const int32_t* num_tokens_post_padded, int64_t num_pairs, int num_experts,
+                     int hidden, int inter, int block_size, int64_t sorted_cap, void* out,
+                     int variant, void* stream) {
+  if (num_pairs == 0) return MOE_I8_OK;
+  if (int rc = check_gemm_common(h_q, w2, sorted_token_ids, expert_ids, num_tokens_post_padded, out,
+                                 num_pairs, num_experts, hidden, inter, block_size, sorted_cap,
+                                 variant))
+    return rc;
+  if (!a_scale || !w2_scale || !topk_weights) return fail(MOE_I8_EINVAL, "null scale pointer");
+  if (!aligned16(w2_scale)) return fail(MOE_I8_EINVAL, "w2_scale must be 16-byte aligned");
+  moe_i8::GemmArgs g{};
+  g.mode = moe_i8::kDown;
+  g.a_q = h_q;
+  g.a_scale = a_scale;
+  g.w = w2;
+  g.w_scale = w2_scale;
+  g.row_weight = topk_weights;
+  g.sorted_token_ids = sorted_token_ids;
+  g.expert_ids = expert_ids;
+  g.num_tokens_post_padded = num_tokens_post_padded;
+  g.num_pairs = num_pairs;
+  g.row_div = 1;
+  g.num_experts = num_experts;
+  g.n = hidden;
+  g.k = inter;
+  g.block_size = block_size;
+  g.sorted_cap = sorted_cap;
+  g.out = out;
+  return run_gemm(g, variant, static_cast<hipStream_t>(stream));
+}
+
+int moe_i8_gemm_acc_i32(const int8_t* a_q, const int8_t* w, const int32_t* sorted_token_ids,
+                        const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
+                        int64_t num_pairs, int row_div, int num_experts, int n, int k,
+                        int block_size, int64_t sorted_cap, int32_t* acc_out, int variant,
+                        void* stream) {
+  if (num_pairs == 0) return MOE_I8_OK;
+  if (int rc = check_gemm_common(a_q, w, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                                 acc_out, num_pairs, num_experts, n, k, block_size, sorted_cap,
+                                 variant))
+    return rc;
+  if (row_div < 1) return fail(MOE_I8_EINVAL, "row_div must be >= 1");
+  moe_i8::GemmArgs g{};
+  g.mode = moe_i8::kAccI32;
+  g.a_q = a_q;
+  g.w = w;
+  g.sorted_token_ids = sorted_token_ids;
+  g.expert_ids = expert_ids;
+  g.num_tokens_post_padded = num_tokens_post_padded;
+  g.num_pairs = num_pairs;
+  g.row_div = row_div;
+  g.num_experts = num_experts;
+  g.n = n;
+  g.k = k;
+  g.block_size = block_size;
+  g.sorted_cap = sorted_cap;
+  g.out = acc_out;
+  return run_gemm(g, variant, static_cast<hipStream_t>(stream));
+}
+
+int moe_i8_sum(const void* in, void* out, int64_t m, int top_k, int hidden, void* stream) {
+  if (m < 0) return fail(MOE_I8_EINVAL, "negative m");
+  if (m == 0) return MOE_I8_OK;
+  if (!in || !out) return fail(MOE_I8_EINVAL, "null pointer");
+  if (top_k < 1) return fail(MOE_I8_EINVAL, "top_k must be >= 1");
+  if (hidden < 8 || hidden % 8) return fail(MOE_I8_EINVAL, "hidden (%d) must be a positive multiple of 8", hidden);
+  if (!aligned16(in) || !aligned16(out)) return fail(MOE_I8_EINVAL, "pointers must be 16-byte aligned");
+  return check_launch(moe_i8::launch_moe_sum(static_cast<const uint16_t*>(in), static_cast<uint16_t*>(out),
+                                             m, top_k, hidden, static_cast<hipStream_t>(stream)),
+                      "moe_sum");
+}
+
+// Workspace layout of moe_i8_fused_experts (every region 256-byte aligned):
+//   x_q i8[M*H] | a1_scale f32[M] | sorted i32[cap] | expert_ids i32[cap/B] | npp i32[1] |
+//   align scratch | act bf16[P*I] | act_q i8[P*I] | a2_scale f32[P] | down_out bf16[P*H]
+namespace {
+struct Carve {
+  int64_t x_q, a1, sorted, eids, npp, align_ws, act, act_q, a2, down, total;
+  int64_t cap, ecap, align_bytes;
+};
+Carve carve(int64_t m, int top_k, int num_experts, int hidden, int inter, int block_size) {
+  Carve c{};
+  const int64_t p = m * top_k;
+  c.cap = moe_i8_sorted_capacity(p, num_experts, block_size);
+  c.ecap = (c.cap + block_size - 1) / block_size;
+  c.align_bytes = moe_i8_align_workspace_bytes(p, num_experts, block_size);
+  int64_t off = 0;
+  auto take = [&](int64_t bytes) {
+    const int64_t at = off;
+    off = align_up(off + bytes, 256);
+    return at;
+  };
+  c.x_q = take(m * hidden);
+  c.a1 = take(m * 4);
+  c.sorted = take(c.cap * 4);
+  c.eids = take(c.ecap * 4);
+  c.npp = take(4);
+  c.align_ws = take(c.align_bytes);
+  c.act = take(p * inter * 2);
+  c.act_q = take(p * inter);
+  c.a2 = take(p * 4);
+  c.down = take(p * hidden * 2);
+  c.total = off;
+  return c;
+}
+}  // namespace
+
+int64_t moe_i8_workspace_bytes(int64_t m, int top_k, int num_experts, int hidden, int inter,
+                               int block_size) {
+  if (m < 0 || top_k < 1 || num_experts < 1 || hidden < 1 || inter < 1 || !valid_block_size(block_size))
+    return -1;
+  return carve(m, top_k, num_experts, hidden, inter, block_size).total;
+}
+
+int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
+                         const float* topk_weights, const int32_t* topk_ids,
+                         const float* w1_scale, const float* w2_scale, void* out, int64_t m,
+                         int top_k, int num_experts, int hidden_size, int inter, int block_size,
+                         void* workspace, int64_t workspace_bytes, int variant, void* stream) {
+  if (m < 0) return fail(MOE_I8_EINVAL, "negative m");
+  if (m == 0) return MOE_I8_OK;
+  if (!hidden || !w1 || !w2 || !topk_weights || !topk_ids || !w1_scale || !w2_scale || !out || !workspace)
+    return fail(MOE_I8_EINVAL, "null pointer");
+  if (top_k < 1 || m * top_k > INT32_MAX - 1) return fail(MOE_I8_EINVAL, "top_k / num_pairs out of range");
+  if (!valid_block_size(block_size)) return fail(MOE_I8_EINVAL, "block_size must be 16, 32, 64 or 128");
+  if (hidden_size < 64 || hidden_size % 64 || inter < 64 || inter % 64)
+    return fail(MOE_I8_EINVAL, "hidden (%d) and inter (%d) must be positive multiples of 64", hidden_size, inter);
+  if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(MOE_I8_EINVAL, "workspace must be 256-byte aligned");
+  const Carve c = carve(m, top_k, num_experts, hidden_size, inter, block_size);
+  if (workspace_bytes < c.total)
+    return fail(MOE_I8_EWORKSPACE, "workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)c.total);
+  char* ws = static_cast<char*>(workspace);
+  int8_t* x_q = reinterpret_cast<int8_t*>(ws + c.x_q);
+  float* a1 = reinterpret_cast<float*>(ws + c.a1);
+  int32_t* sorted = reinterpret_cast<int32_t*>(ws + c.sorted);
+  int32_t* eids = reinterpret_cast<int32_t*>(ws + c.eids);
+  int32_t* npp = reinterpret_cast<int32_t*>(ws + c.npp);
+  void* act = ws + c.act;
+  int8_t* act_q = reinterpret_cast<int8_t*>(ws + c.act_q);
+  float* a2 = reinterpret_cast<float*>(ws + c.a2);
+  void* down = ws + c.down;
+  const int64_t p = m * top_k;
+
+  if (int rc = moe_i8_quant_rows(hidden, MOE_I8_DTYPE_BF16, m, hidden_size, hidden_size, nullptr, 1, m,
+                                 x_q, a1, stream))
+    return rc;
+  if (int rc = moe_i8_align_block_size(topk_ids, p, num_experts, block_size, sorted, c.cap, eids, c.ecap,
+                                       npp, ws + c.align_ws, c.align_bytes, stream))
+    return rc;
+  if (int rc = moe_i8_gemm_gate_up_silu(x_q, a1, w1, w1_scale, sorted, eids, npp, p, top_k, num_experts,
+                                        hidden_size, inter, block_size, c.cap, act, variant, stream))
+    return rc;
+  if (int rc = moe_i8_quant_rows(act, MOE_I8_DTYPE_BF16, p, inter, inter, nullptr, 1, p, act_q, a2, stream))
+    return rc;
+  if (int rc = moe_i8_gemm_down(act_q, a2, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
+                                hidden_size, inter, block_size, c.cap, down, variant, stream))
+    return rc;
+  return moe_i8_sum(down, out, m, top_k, hidden_size, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,96 @@
+// Shared device helpers and launcher declarations for the gfx950 INT8 MoE kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace moe_i8 {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int kWave = 64;
+constexpr int kMaxExperts = 1024;  // == MOE_I8_MAX_EXPERTS
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// fp32 -> bf16 bits, round to nearest even; NaN stays a quiet NaN.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+__device__ __forceinline__ float round_to_bf16(float f) {
+  return bf16_bits_to_f32(f32_to_bf16_bits(f));
+}
+
+// SiLU-gated product with the rounding points of a bf16 silu_and_mul kernel:
+// silu in fp32, rounded to bf16, times up in fp32, rounded to bf16.
+__device__ __forceinline__ uint32_t silu_mul_bf16_bits(float gate, float up) {
+  float s = round_to_bf16(gate / (1.0f + expf(-gate)));
+  return f32_to_bf16_bits(s * up);
+}
+
+// ---- launchers (defined one per .hip file; all asynchronous on `stream`) ----
+
+struct AlignArgs {
+  const int32_t* topk_ids;
+  int64_t num_pairs;
+  int num_experts;
+  int block_size;
+  int32_t* sorted_token_ids;
+  int64_t sorted_cap;
+  int32_t* expert_ids;
+  int64_t expert_cap;
+  int32_t* num_tokens_post_padded;
+  int32_t* workspace;
+};
+int64_t align_workspace_ints(int64_t num_pairs, int num_experts);
+hipError_t launch_align(const AlignArgs& a, hipStream_t stream);
+
+struct QuantArgs {
+  const uint16_t* x;  // bf16 bits
+  int64_t src_rows;
+  int cols;
+  int64_t row_stride;
+  const int32_t* gather;
+  int gather_div;
+  int64_t rows;
+  int8_t* q;
+  float* scale;
+};
+hipError_t launch_quant_rows(const QuantArgs& a, hipStream_t stream);
+
+enum GemmMode { kGateUpSilu = 0, kDown = 1, kAccI32 = 2 };
+
+struct GemmArgs {
+  int mode;
+  const int8_t* a_q;      // [*, K] activations (int8)
+  const float* a_scale;   // per activation row
+  const int8_t* w;        // [E, N, K]
+  const float* w_scale;   // [E, N]
+  const float* row_weight;  // [P] routed weights (down) or null
+  const int32_t* sorted_token_ids;
+  const int32_t* expert_ids;
+  const int32_t* num_tokens_post_padded;
+  int64_t num_pairs;
+  int row_div;  // activation row of pair t is t / row_div
+  int num_experts;
+  int n;  // weight rows per expert (2I for gate_up, H for down)
+  int k;  // reduction length
+  int block_size;
+  int64_t sorted_cap;
+  void* out;  // bf16 [P, I] | bf16 [P, H] | int32 [P, N]
+};
+hipError_t launch_gemm_stream(const GemmArgs& a, hipStream_t stream);
+hipError_t launch_gemm_tile(const GemmArgs& a, hipStream_t stream);
+bool gemm_tile_supports(const GemmArgs& a);
+
+hipError_t launch_moe_sum(const uint16_t* in, uint16_t* out, int64_t m, int top_k, int hidden,
+                          hipStream_t stream);
+
+}  // namespace moe_i8

@@ -1,0 +1,139 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports every symbol the header
+declares, validates its arguments with error codes (no launch happens), and the Python wrappers
+raise instead of falling back."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def _declared_symbols():
+    text = (ROOT / "include" / "moe_i8.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(moe_i8_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(pra):
+    lib = pra._abi.load()
+    declared = _declared_symbols()
+    assert len(declared) >= 12
+    assert sorted(pra._abi.SIGNATURES) == declared
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.moe_i8_version() >= 1
+
+
+def test_capacity_and_workspace_formulas(pra):
+    lib = pra._abi.load()
+    assert lib.moe_i8_sorted_capacity(12, 5, 4) == 12 + 5 * 3
+    assert lib.moe_i8_sorted_capacity(128, 128, 64) == 128 * 64  # fewer pairs than experts: P*B
+    assert lib.moe_i8_sorted_capacity(65536, 128, 64) == 65536 + 128 * 63
+    assert lib.moe_i8_sorted_capacity(0, 8, 64) == 0
+    assert lib.moe_i8_align_workspace_bytes(1024, 128, 64) == 0
+    big = lib.moe_i8_align_workspace_bytes(131072, 256, 64)
+    assert big == 4 * (128 * 256 + 257)
+    ws = lib.moe_i8_workspace_bytes(16, 8, 128, 2048, 768, 64)
+    P = 128
+    assert ws >= 16 * 2048 + P * 768 * 3 + P * 2048 * 2 and ws % 256 == 0
+    assert lib.moe_i8_workspace_bytes(16, 8, 128, 2048, 768, 48) == -1
+
+
+def test_c_abi_rejects_bad_arguments_without_launching(pra):
+    abi = pra._abi
+    lib = abi.load()
+    buf = (ctypes.c_int32 * 1024)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    err = lambda: lib.moe_i8_last_error().decode()
+    # align: null outputs, bad block size, too many experts, capacity too small
+    assert lib.moe_i8_align_block_size(p, 8, 4, 64, None, 260, p, 5, p, None, 0, None) == abi.EINVAL
+    assert lib.moe_i8_align_block_size(p, 8, 4, 48, p, 260, p, 5, p, None, 0, None) == abi.EINVAL
+    assert "block_size" in err()
+    assert lib.moe_i8_align_block_size(p, 8, 2000, 64, p, 10**6, p, 10**5, p, None, 0, None) == abi.EINVAL
+    assert lib.moe_i8_align_block_size(p, 8, 4, 64, p, 10, p, 5, p, None, 0, None) == abi.EWORKSPACE
+    assert lib.moe_i8_align_block_size(p, 20000, 4, 64, p, 20000 + 4 * 63, p, 400, p, None, 0, None) == abi.EWORKSPACE
+    assert "workspace" in err()
+    # quant: dtype, cols, stride, alignment
+    assert lib.moe_i8_quant_rows(p, 7, 4, 64, 64, None, 1, 4, p, p, None) == abi.EUNSUPPORTED
+    assert lib.moe_i8_quant_rows(p, 0, 4, 60, 64, None, 1, 4, p, p, None) == abi.EINVAL
+    assert lib.moe_i8_quant_rows(p, 0, 4, 64, 32, None, 1, 4, p, p, None) == abi.EINVAL
+    assert lib.moe_i8_quant_rows(None, 0, 4, 64, 64, None, 1, 4, p, p, None) == abi.EINVAL
+    assert lib.moe_i8_quant_rows(p, 0, 4, 64, 64, None, 1, 0, p, p, None) == abi.OK  # zero rows: no-op
+    # gemm: K not multiple of 64, N not multiple of 16, unknown variant, null
+    base = dict(num_pairs=8, top_k=2, E=4, H=128, I=64, B=64, cap=8 + 4 * 63)
+    call = lambda H=128, I=64, variant=0, x=p: lib.moe_i8_gemm_gate_up_silu(
+        x, p, p, p, p, p, p, base["num_pairs"], 2, 4, H, I, 64, base["cap"], p, variant, None
+    )
+    assert call(H=96) == abi.EINVAL
+    assert call(I=24) == abi.EINVAL
+    assert call(variant=9) == abi.EINVAL
+    assert call(x=None) == abi.EINVAL
+    assert lib.moe_i8_gemm_down(p, p, p, p, p, p, p, p, 8, 4, 128, 100, 64, 260, p, 0, None) == abi.EINVAL
+    assert lib.moe_i8_gemm_acc_i32(p, p, p, p, p, 8, 0, 4, 128, 128, 64, 260, p, 0, None) == abi.EINVAL
+    # sum / fused driver
+    assert lib.moe_i8_sum(p, p, 4, 0, 64, None) == abi.EINVAL
+    assert lib.moe_i8_sum(p, p, 4, 2, 20, None) == abi.EINVAL
+    assert lib.moe_i8_sum(None, None, 0, 2, 64, None) == abi.OK
+    assert lib.moe_i8_fused_experts(p, p, p, p, p, p, p, p, 4, 2, 4, 128, 64, 64, None, 0, 0, None) == abi.EINVAL
+    assert lib.moe_i8_fused_experts(p, p, p, p, p, p, p, p, 4, 2, 4, 100, 64, 64, p, 1 << 30, 0, None) == abi.EINVAL
+
+
+def test_python_wrappers_refuse_cpu_tensors_and_unsupported_modes(pra):
+    x = torch.zeros((4, 128), dtype=torch.bfloat16)
+    w1 = torch.zeros((2, 128, 128), dtype=torch.int8)
+    w2 = torch.zeros((2, 128, 64), dtype=torch.int8)
+    tw = torch.ones((4, 1))
+    ids = torch.zeros((4, 1), dtype=torch.int32)
+    s1, s2 = torch.ones((2, 128)), torch.ones((2, 128))
+    kw = dict(use_int8_w8a8=True, per_channel_quant=True, w1_scale=s1, w2_scale=s2)
+    with pytest.raises(ValueError, match="GPU tensor"):
+        pra.fused_experts(x, w1, w2, tw, ids, **kw)
+    with pytest.raises(ValueError, match="GPU tensor"):
+        pra.moe_align_block_size(ids, 64, 2)
+    with pytest.raises(ValueError, match="GPU tensor"):
+        pra.per_token_quant_int8(x)
+    with pytest.raises(NotImplementedError):
+        pra.fused_experts(x, w1, w2, tw, ids, w1_scale=s1, w2_scale=s2)  # not int8
+    with pytest.raises(NotImplementedError):
+        pra.fused_experts(x, w1, w2, tw, ids, **{**kw, "per_channel_quant": False})
+    with pytest.raises(NotImplementedError):
+        pra.fused_experts(x, w1, w2, tw, ids, activation="gelu", **kw)
+    with pytest.raises(NotImplementedError):
+        pra.fused_experts(x, w1, w2, tw, ids, expert_map=torch.zeros(2), **kw)
+    with pytest.raises(NotImplementedError):
+        pra.fused_experts(x, w1, w2, tw, ids, block_shape=[128, 128], **kw)
+    with pytest.raises(NotImplementedError):
+        pra.fused_experts(x, w1, w2, tw, ids, apply_router_weight_on_input=True, **kw)
+    with pytest.raises(NotImplementedError):
+        pra.moe_align_block_size(ids, 64, 2, expert_map=torch.zeros(2))
+
+
+def test_fused_experts_signature_is_vllms(pra):
+    import inspect
+
+    params = list(inspect.signature(pra.fused_experts).parameters)
+    assert params[:5] == ["hidden_states", "w1", "w2", "topk_weights", "topk_ids"]
+    for name in ("inplace", "activation", "apply_router_weight_on_input", "use_int8_w8a8", "per_channel_quant",
+                 "global_num_experts", "expert_map", "w1_scale", "w2_scale", "a1_scale", "a2_scale", "block_shape"):
+        assert name in params
+    assert list(inspect.signature(pra.moe_align_block_size).parameters) == [
+        "topk_ids", "block_size", "num_experts", "expert_map", "pad_sorted_ids"]
+    assert list(inspect.signature(pra.moe_sum).parameters) == ["input", "output"]
+
+
+def test_vllm_plugin_is_noop_without_vllm(pra, monkeypatch):
+    monkeypatch.setenv(pra.vllm_plugin.ENV_FLAG, "1")
+    assert pra.vllm_plugin.register() is False
+    monkeypatch.setenv(pra.vllm_plugin.ENV_FLAG, "0")
+    assert pra.vllm_plugin.register() is False
+
+
+def test_missing_library_fails_loudly(pra, monkeypatch, tmp_path):
+    monkeypatch.setattr(pra._abi, "_lib", None)
+    monkeypatch.setattr(pra._abi, "LIB_PATH", tmp_path / "libmoe_i8.so")
+    with pytest.raises(ImportError, match="no CPU or PyTorch fallback"):
+        pra._abi.load()

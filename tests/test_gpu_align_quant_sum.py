@@ -1,0 +1,172 @@
+"""GPU parity (bit-exact): moe_align_block_size, per_token_quant_int8 and moe_sum through the C-ABI
+against the CPU oracle and the committed known-answer vectors."""
+
+import pytest
+import torch
+
+from _util import inputs_mod
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _check_align(pra, oracle, ids_cpu, B, E):
+    P = ids_cpu.numel()
+    s, e, npp = pra.moe_align_block_size(ids_cpu.to(DEV), B, E)
+    torch.cuda.synchronize()
+    so, eo, nppo = oracle.moe_align_block_size(ids_cpu.clamp(-1, E), B, E)  # out-of-range handled by caller
+    n = int(nppo)
+    assert int(npp.cpu()) == n, (int(npp.cpu()), n)
+    assert s.numel() == min(P + E * (B - 1), P * B) and e.numel() == (s.numel() + B - 1) // B
+    assert torch.equal(s.cpu()[:n], so[:n])
+    assert torch.equal(e.cpu()[: n // B], eo[: n // B])
+    assert bool((s.cpu()[n:] == P).all()) and bool((e.cpu()[n // B :] == -1).all())
+    return s, e, npp
+
+
+def test_align_known_answer(pra, oracle, golden):
+    g = golden["align_docstring_example"]
+    ids = torch.tensor(g["topk_ids"], dtype=torch.int32)
+    # block 4 is not a GEMM block size; the docstring case is checked at block 16 through its counts
+    s, e, npp = pra.moe_align_block_size(ids.to(DEV), 16, g["num_experts"])
+    s, e = s.cpu(), e.cpu()
+    assert int(npp.cpu()) == 64 and e[:4].tolist() == g["expert_ids_prefix"]
+    for j, members in enumerate(([3, 6, 9], [0, 4, 10], [1, 7, 11], [2, 5, 8])):
+        assert s[16 * j : 16 * j + 3].tolist() == members and bool((s[16 * j + 3 : 16 * j + 16] == 12).all())
+
+
+@pytest.mark.parametrize("shape_name,M", [
+    ("toy", 256), ("qwen3-30b-a3b", 1), ("qwen3-30b-a3b", 16), ("qwen3-30b-a3b", 128),
+    ("qwen3-30b-a3b", 1024), ("qwen3-30b-a3b", 8192), ("glm-4.5-air", 32), ("glm-4.5-air", 512),
+    ("glm-4.5-air", 4096), ("deepseek-v3", 8), ("deepseek-v3", 64), ("deepseek-v3", 2048),
+    ("deepseek-v3", 16384),
+])
+def test_align_baseline_routings(pra, oracle, shape_name, M):
+    im = inputs_mod()
+    shape = im.SHAPES[shape_name]
+    _, ids = im.route(shape, M, torch.Generator().manual_seed(M))
+    _check_align(pra, oracle, ids, 64, shape.E_total)
+
+
+@pytest.mark.parametrize("B", [16, 32, 64, 128])
+@pytest.mark.parametrize("E,P", [(1, 1), (1, 700), (3, 2), (8, 8191), (8, 8193), (257, 9000), (1024, 5000), (1024, 70000)])
+def test_align_block_sizes_and_extremes(pra, oracle, B, E, P):
+    ids = torch.randint(0, E, (P, 1), generator=torch.Generator().manual_seed(P + E), dtype=torch.int32)
+    _check_align(pra, oracle, ids, B, E)
+
+
+def test_align_edge_cases(pra, oracle):
+    _check_align(pra, oracle, torch.tensor([[0], [2]], dtype=torch.int32), 16, 3)  # unused expert
+    _check_align(pra, oracle, torch.full((100, 8), 7, dtype=torch.int32), 64, 128)  # one hot expert
+    _check_align(pra, oracle, torch.full((20000, 1), 5, dtype=torch.int32), 64, 8)  # same, multi-launch
+    _check_align(pra, oracle, torch.arange(4, dtype=torch.int32).repeat_interleave(64).reshape(-1, 1), 64, 4)
+    s, e, npp = pra.moe_align_block_size(torch.zeros((0, 8), dtype=torch.int32, device=DEV), 64, 128)
+    assert int(npp.cpu()) == 0 and s.numel() == 0
+
+
+def test_align_int64_ids_and_out_of_range_ignored(pra, oracle):
+    ids = torch.randint(0, 16, (333, 4), generator=torch.Generator().manual_seed(1), dtype=torch.int64)
+    _check_align(pra, oracle, ids.to(torch.int32), 64, 16)
+    s64, e64, n64 = pra.moe_align_block_size(ids.to(DEV), 64, 16)
+    s32, e32, n32 = pra.moe_align_block_size(ids.to(torch.int32).to(DEV), 64, 16)
+    assert torch.equal(s64, s32) and torch.equal(e64, e32) and torch.equal(n64, n32)
+    bad = ids.to(torch.int32).clone()
+    bad[5, 1], bad[9, 0] = 16, -3
+    s, e, npp = pra.moe_align_block_size(bad.to(DEV), 64, 16)
+    keep = (bad.reshape(-1) >= 0) & (bad.reshape(-1) < 16)
+    real = s.cpu()[s.cpu() < bad.numel()]
+    assert sorted(real.tolist()) == torch.nonzero(keep).reshape(-1).tolist()
+
+
+def test_align_is_deterministic(pra):
+    im = inputs_mod()
+    _, ids = im.route(im.SHAPES["deepseek-v3"], 4096, torch.Generator().manual_seed(0))
+    ids = ids.to(DEV)
+    first = pra.moe_align_block_size(ids, 64, 256)
+    for _ in range(5):
+        again = pra.moe_align_block_size(ids, 64, 256)
+        assert all(torch.equal(a, b) for a, b in zip(first, again))
+
+
+# ------------------------------------------------------------------------------------ quant
+def test_quant_known_answer(pra, golden):
+    g = golden["quant_ties"]
+    x = torch.tensor([g["x"], [0.0] * 8], dtype=torch.bfloat16, device=DEV)
+    q, s = pra.per_token_quant_int8(x)
+    assert q.cpu()[0].tolist() == g["q_half_away"] and s.shape == (2, 1)
+    assert float(s.cpu()[0, 0]) == g["scale"]
+    assert q.cpu()[1].tolist() == [0] * 8
+    assert float(s.cpu()[1, 0]) == pytest.approx(g["zero_row_scale"], rel=1e-6)
+
+
+@pytest.mark.parametrize("rows,cols", [
+    (1, 8), (3, 64), (256, 1024), (16, 2048), (1031, 768), (77, 2816), (64, 1408), (33, 7168),
+    (5, 4096), (9, 8192), (4, 16384), (3, 9000),
+])
+def test_quant_bit_exact(pra, oracle, rows, cols):
+    g = torch.Generator().manual_seed(rows * 131 + cols)
+    x = (torch.randn((rows, cols), generator=g) * torch.rand((rows, 1), generator=g) * 8).to(torch.bfloat16)
+    if rows > 2:
+        x[1] = 0
+    q, s = pra.per_token_quant_int8(x.to(DEV))
+    qo, so = oracle.per_token_quant_int8(x)
+    assert torch.equal(s.cpu(), so), float((s.cpu() - so).abs().max())
+    assert torch.equal(q.cpu(), qo), int((q.cpu() != qo).sum())
+
+
+def test_quant_3d_and_full_size(pra, oracle):
+    x = torch.randn((4, 8, 768), generator=torch.Generator().manual_seed(2)).to(torch.bfloat16)
+    q, s = pra.per_token_quant_int8(x.to(DEV))
+    qo, so = oracle.per_token_quant_int8(x)
+    assert q.shape == x.shape and s.shape == (4, 8, 1)
+    assert torch.equal(q.cpu(), qo) and torch.equal(s.cpu(), so)
+    # baseline maximum: 16384 x 7168 activations
+    x = torch.randn((16384, 7168), generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    q, s = pra.per_token_quant_int8(x.to(DEV))
+    qo, so = oracle.per_token_quant_int8(x)
+    assert torch.equal(s.cpu(), so) and torch.equal(q.cpu(), qo)
+
+
+def test_quant_gather_through_c_abi(pra, oracle):
+    """Output row r = quantised input row gather[r] // div; sentinel rows come out as zeros."""
+    abi = pra._abi
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn((10, 512), generator=g).to(torch.bfloat16)
+    idx = torch.tensor([6, 7, 0, 19, 20, 3, 40, 2], dtype=torch.int32)  # //2 -> 3,3,0,9,10(sentinel),1,20(sentinel),1
+    xd, idxd = x.to(DEV), idx.to(DEV)
+    q = torch.full((8, 512), 99, dtype=torch.int8, device=DEV)
+    s = torch.zeros((8,), dtype=torch.float32, device=DEV)
+    abi.check(abi.load().moe_i8_quant_rows(xd.data_ptr(), 0, 10, 512, 512, idxd.data_ptr(), 2, 8, q.data_ptr(),
+                                            s.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    qo, so = oracle.per_token_quant_int8(x)
+    for r, src in enumerate((idx // 2).tolist()):
+        if src < 10:
+            assert torch.equal(q.cpu()[r], qo[src]) and float(s.cpu()[r]) == float(so[src, 0])
+        else:
+            assert bool((q.cpu()[r] == 0).all())
+
+
+# ------------------------------------------------------------------------------------ moe_sum
+@pytest.mark.parametrize("M,k,H", [(1, 1, 8), (256, 2, 1024), (7, 3, 64), (5, 4, 4096), (1024, 8, 2048),
+                                   (32, 9, 4096), (64, 8, 7168), (3, 16, 128)])
+def test_moe_sum_bit_exact(pra, oracle, M, k, H):
+    g = torch.Generator().manual_seed(M + k + H)
+    c3 = torch.randn((M, k, H), generator=g).to(torch.bfloat16)
+    out = torch.empty((M, H), dtype=torch.bfloat16, device=DEV)
+    pra.moe_sum(c3.to(DEV), out)
+    want = oracle.moe_sum(c3)
+    assert torch.equal(out.cpu(), want), float((out.cpu().float() - want.float()).abs().max())
+
+
+def test_moe_sum_reference_known_answer(pra, golden):
+    """Combine convention of the reference dispatcher test (values exactly representable in bf16
+    are used: x^2*(e+1) with small integer x, weights 0.5/0.25, so no rounding occurs)."""
+    x = (torch.arange(12, dtype=torch.float32) % 4).reshape(4, 3)
+    sel = torch.tensor(golden["dispatcher_known_answer"]["selected"])
+    w = torch.tensor([[0.5, 0.25], [0.25, 0.5], [0.5, 0.5], [0.25, 0.25]])
+    c3 = torch.zeros((4, 2, 8))
+    c3[:, :, :3] = x.square()[:, None, :] * (sel[:, :, None] + 1) * w[:, :, None]
+    out = torch.empty((4, 8), dtype=torch.bfloat16, device=DEV)
+    pra.moe_sum(c3.to(torch.bfloat16).to(DEV), out)
+    want = c3.sum(1)
+    assert torch.equal(out.cpu().float(), want)

@@ -1,0 +1,111 @@
+"""GPU parity for the grouped int8 GEMMs through the C-ABI: int32 accumulators bit-exact, the down
+epilogue bit-exact, the SiLU-gated epilogue to within one bf16 step (the only difference is the
+last bit of expf)."""
+
+import pytest
+import torch
+
+from _util import bf16_ulp_diff, inputs_mod
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+VARIANTS = ["stream", "tile"]
+
+
+def _problem(oracle, E, k, H, I, M, seed, B=64, routing="softmax"):
+    im = inputs_mod()
+    shape = im.LayerShape("t", E=E, k=k, H=H, I=I, routing=routing)
+    inp = im.make_inputs(shape, M, seed=seed)
+    st = oracle.fused_experts_staged(inp.hidden_states, inp.w1, inp.w2, inp.topk_weights, inp.topk_ids,
+                                     inp.w1_scale, inp.w2_scale, B)
+    return inp, st
+
+
+def _routing_on_gpu(pra, inp, B):
+    return pra.moe_align_block_size(inp.topk_ids.to(DEV), B, inp.w1.shape[0])
+
+
+def _skip_if_unsupported(pra, fn):
+    try:
+        return fn()
+    except pra._abi.MoeI8Error as exc:
+        if exc.code == pra._abi.EUNSUPPORTED:
+            pytest.skip(str(exc))
+        raise
+
+
+SHAPES = [
+    # E, k, H, I, M, B
+    (4, 2, 128, 64, 5, 16),
+    (8, 2, 256, 192, 96, 64),
+    (8, 2, 1024, 2816, 256, 64),     # toy layer of the baseline
+    (128, 8, 2048, 768, 16, 64),     # Qwen3-30B-A3B decode
+    (128, 8, 2048, 768, 300, 64),
+    (16, 4, 1408, 448, 200, 32),     # K = 22 * 64: exercises the unroll tail
+    (3, 1, 64, 64, 700, 128),        # one 16-channel tile, block 128
+    (32, 8, 512, 320, 64, 64),
+]
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("E,k,H,I,M,B", SHAPES)
+def test_int32_accumulators_bit_exact(pra, oracle, variant, E, k, H, I, M, B):
+    inp, st = _problem(oracle, E, k, H, I, M, seed=E + M, B=B)
+    s, e, npp = _routing_on_gpu(pra, inp, B)
+    P = M * k
+    acc1 = _skip_if_unsupported(pra, lambda: pra.gemm_acc_i32(
+        st["x_q"].to(DEV), inp.w1.to(DEV), s, e, npp, k, B, P, variant))
+    assert torch.equal(acc1.cpu(), st["acc1"]), int((acc1.cpu() != st["acc1"]).sum())
+    acc2 = pra.gemm_acc_i32(st["h_q"].to(DEV), inp.w2.to(DEV), s, e, npp, 1, B, P, variant)
+    assert torch.equal(acc2.cpu(), st["acc2"]), int((acc2.cpu() != st["acc2"]).sum())
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_accumulators_extreme_values(pra, oracle, variant):
+    """All operands at +-127 with K=7168: the largest magnitude the path can produce."""
+    E, k, H, N, M, B = 2, 1, 7168, 64, 40, 64
+    a = torch.full((M, H), 127, dtype=torch.int8)
+    a[::2] = -127
+    w = torch.full((E, N, H), -127, dtype=torch.int8)
+    w[1, ::3] = 127
+    ids = (torch.arange(M, dtype=torch.int32) % E).reshape(M, 1)
+    s, e, npp = pra.moe_align_block_size(ids.to(DEV), B, E)
+    acc = _skip_if_unsupported(pra, lambda: pra.gemm_acc_i32(a.to(DEV), w.to(DEV), s, e, npp, 1, B, M, variant))
+    want = oracle.grouped_int_gemm(a, w, ids, 1)
+    assert int(want.abs().max()) == 127 * 127 * 7168
+    assert torch.equal(acc.cpu(), want)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("E,k,H,I,M,B", SHAPES)
+def test_down_gemm_epilogue_bit_exact(pra, oracle, variant, E, k, H, I, M, B):
+    inp, st = _problem(oracle, E, k, H, I, M, seed=E + M + 1, B=B)
+    s, e, npp = _routing_on_gpu(pra, inp, B)
+    out = _skip_if_unsupported(pra, lambda: pra.gemm_down(
+        st["h_q"].to(DEV), st["a2_scale"].to(DEV), inp.w2.to(DEV), inp.w2_scale.to(DEV),
+        inp.topk_weights.to(DEV), s, e, npp, B, variant))
+    want = st["cache3"].reshape(M * k, H)
+    assert torch.equal(out.cpu(), want), int((out.cpu() != want).sum())
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("E,k,H,I,M,B", SHAPES)
+def test_gate_up_silu_within_one_bf16_step(pra, oracle, variant, E, k, H, I, M, B):
+    inp, st = _problem(oracle, E, k, H, I, M, seed=E + M + 2, B=B)
+    s, e, npp = _routing_on_gpu(pra, inp, B)
+    act = _skip_if_unsupported(pra, lambda: pra.gemm_gate_up_silu(
+        st["x_q"].to(DEV), st["a1_scale"].to(DEV), inp.w1.to(DEV), inp.w1_scale.to(DEV), s, e, npp,
+        k, B, M * k, variant))
+    d = bf16_ulp_diff(act, st["cache2"])
+    assert int(d.max()) <= 1, int(d.max())
+    assert float((d > 0).float().mean()) < 1e-3, float((d > 0).float().mean())
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_gemm_is_deterministic(pra, oracle, variant):
+    inp, st = _problem(oracle, 16, 4, 512, 256, 333, seed=7)
+    s, e, npp = _routing_on_gpu(pra, inp, 64)
+    args = (st["x_q"].to(DEV), st["a1_scale"].to(DEV), inp.w1.to(DEV), inp.w1_scale.to(DEV), s, e, npp, 4, 64, 333 * 4)
+    first = _skip_if_unsupported(pra, lambda: pra.gemm_gate_up_silu(*args, variant))
+    for _ in range(3):
+        assert torch.equal(first, pra.gemm_gate_up_silu(*args, variant))
