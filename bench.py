@@ -1,0 +1,230 @@
+#!/usr/bin/env python3
+"""Benchmark of the gfx950 INT8 W8A8 fused-MoE layer on one MI355X.
+
+A step is one ``fused_experts`` call (quant → align → gate_up GEMM + SiLU·mul → quant → down GEMM →
+combine) on one batch of M tokens of the Qwen3-30B-A3B-shaped layer (E=128, top-8, H=2048, I=768,
+moe_align block 64), inputs resident in HBM.  The headline value is tokens/s at ``--m`` (default
+8192, the prefill point); ``sweep`` repeats the measurement at M = 16, 128, 1024, 8192 and reports
+layer-level INT8 TOP/s and HBM GB/s from the algorithmic work of the sampled routing.  Successive
+steps rotate over several independent weight copies so that no step finds its weights in the
+256 MB last-level cache.
+
+Prints one JSON line.  ``roofline`` describes the dominant kernel (the gate_up GEMM), timed with
+events on the launch stream; ``cpu_baseline`` is the torch-native W8A8 MoE of the CPU oracle timed
+on the host cores (a reported baseline, not a target).
+"""
+
+from __future__ import annotations
+
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+PEAK_INT8_OPS = 5.0e15  # MI355X dense INT8 MFMA, op/s
+PEAK_HBM_BPS = 8.0e12  # MI355X HBM3E, byte/s
+SWEEP_M = (16, 128, 1024, 8192)
+
+
+def _profile_traffic(kernel: str, M: int):
+    """HBM bytes per launch measured with rocprofv3 --pmc, when a summary for this kernel and batch
+    size has been recorded in profiles/traffic.json; otherwise None."""
+    path = ROOT / "profiles" / "traffic.json"
+    if not path.exists():
+        return None
+    try:
+        return json.loads(path.read_text()).get(f"{kernel}@M={M}")
+    except (ValueError, OSError):
+        return None
+
+
+def build_workload(pkg, torch, shape_name: str, M: int, copies: int, seed: int):
+    inputs = pkg.inputs
+    shape = inputs.SHAPES[shape_name]
+    base = inputs.make_inputs(shape, M, seed=seed)
+    dev = base.to("cuda:0")
+    weights = [(dev.w1, dev.w2, dev.w1_scale, dev.w2_scale)]
+    for c in range(1, copies):
+        # independent copies: same distribution, different bits (a roll along the expert axis)
+        weights.append(tuple(t.roll(c, 0).contiguous() for t in weights[0]))
+    return shape, base, dev, weights
+
+
+def time_layer(pkg, torch, dev, weights, steps: int, warmup: int, variant: str) -> float:
+    def step(i):
+        w1, w2, s1, s2 = weights[i % len(weights)]
+        return pkg.fused_experts(dev.hidden_states, w1, w2, dev.topk_weights, dev.topk_ids,
+                                 use_int8_w8a8=True, per_channel_quant=True, w1_scale=s1, w2_scale=s2,
+                                 gemm_variant=variant)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def time_gate_up_kernel(pkg, torch, shape, dev, weights, steps: int, warmup: int, variant: str) -> float:
+    """Average duration (s) of the gate_up GEMM launch, from event pairs on the launch stream."""
+    M, k = dev.topk_ids.shape
+    x_q, a1 = pkg.per_token_quant_int8(dev.hidden_states)
+    s, e, npp = pkg.moe_align_block_size(dev.topk_ids, 64, shape.E_total)
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    for i in range(warmup):
+        w1, _, s1, _ = weights[i % len(weights)]
+        pkg.gemm_gate_up_silu(x_q, a1, w1, s1, s, e, npp, k, 64, M * k, variant)
+    torch.cuda.synchronize()
+    for i in range(steps):
+        w1, _, s1, _ = weights[i % len(weights)]
+        starts[i].record()
+        pkg.gemm_gate_up_silu(x_q, a1, w1, s1, s, e, npp, k, 64, M * k, variant)
+        stops[i].record()
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in zip(starts, stops)) / steps * 1e-3
+
+
+def gate_up_work(shape, M: int, topk_ids):
+    """Algorithmic work of one gate_up GEMM launch: int8 ops, and HBM bytes (weights and channel
+    scales of the routed-to experts, int8 activations and their scales in, bf16 activations out)."""
+    import torch
+
+    k = topk_ids.shape[1]
+    P = M * k
+    n_act = int(torch.unique(topk_ids).numel())
+    ops = 4 * P * shape.I * shape.H
+    nbytes = n_act * (2 * shape.I * shape.H + 8 * shape.I) + M * shape.H + 4 * M + 2 * P * shape.I + 4 * P
+    return ops, nbytes, n_act
+
+
+def cpu_baseline(oracle, torch, base, sample_m: int) -> dict:
+    m = min(sample_m, base.hidden_states.shape[0])
+    args = (base.hidden_states[:m], base.w1, base.w2, base.topk_weights[:m], base.topk_ids[:m],
+            base.w1_scale, base.w2_scale)
+    oracle.native_w8a8_moe(*args)  # warm-up
+    best = float("inf")
+    for _ in range(2):
+        t0 = time.perf_counter()
+        oracle.native_w8a8_moe(*args)
+        best = min(best, time.perf_counter() - t0)
+    return {
+        "value": m / best,
+        "unit": "tokens/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"first {m} tokens of the same seeded workload, torch-native W8A8 MoE of the oracle, "
+                  f"best of 2 after 1 warm-up ({best:.2f} s per pass; os.cpu_count()={os.cpu_count()})",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--m", type=int, default=8192, help="tokens per step of the headline measurement")
+    ap.add_argument("--shape", default="qwen3-30b-a3b")
+    ap.add_argument("--variant", default="auto", choices=["auto", "stream", "tile"])
+    ap.add_argument("--weight-copies", type=int, default=4)
+    ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--cpu-sample", type=int, default=4096, help="tokens of the workload the CPU baseline runs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    pkg = importlib.import_module("prime_rl_amd")
+    pkg._abi.load()  # fails loudly if the HIP library is not built
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+
+    sweep = []
+    headline = None
+    ms = [args.m] if args.no_sweep else sorted(set(SWEEP_M) | {args.m})
+    base_headline = None
+    for M in ms:
+        shape, base, dev, weights = build_workload(pkg, torch, args.shape, M, args.weight_copies, seed=M)
+        t_layer = time_layer(pkg, torch, dev, weights, args.steps, args.warmup, args.variant)
+        t_k = time_gate_up_kernel(pkg, torch, shape, dev, weights, args.steps, args.warmup, args.variant)
+        ops_layer = pkg.inputs.algorithmic_ops(shape, M)
+        bytes_layer = pkg.inputs.algorithmic_bytes(shape, M, base.topk_ids)
+        k_ops, k_bytes, n_act = gate_up_work(shape, M, base.topk_ids)
+        hbm_bound = (bytes_layer / PEAK_HBM_BPS) >= (ops_layer / PEAK_INT8_OPS)
+        if hbm_bound:
+            roof = {"bound": "hbm", "achieved": k_bytes / t_k / 1e9, "peak": PEAK_HBM_BPS / 1e9, "unit": "GB/s"}
+        else:
+            roof = {"bound": "mfma", "achieved": k_ops / t_k / 1e12, "peak": PEAK_INT8_OPS / 1e12, "unit": "TFLOP/s",
+                    "note": "int8 TOP/s against the dense INT8 MFMA peak"}
+        roof["frac"] = roof["achieved"] / roof["peak"]
+        roof["kernel"] = "gemm gate_up + SiLU*mul"
+        roof["kernel_us"] = t_k * 1e6
+        roof["traffic"] = _profile_traffic("gate_up", M)
+        point = {
+            "M": M,
+            "tokens_per_s": M / t_layer,
+            "ms_per_step": t_layer * 1e3,
+            "n_active_experts": n_act,
+            "layer_int8_tops": ops_layer / t_layer / 1e12,
+            "layer_mfma_frac": ops_layer / t_layer / PEAK_INT8_OPS,
+            "layer_hbm_gbps": bytes_layer / t_layer / 1e9,
+            "layer_hbm_frac": bytes_layer / t_layer / PEAK_HBM_BPS,
+            "roofline": roof,
+        }
+        sweep.append(point)
+        if M == args.m:
+            headline, base_headline = point, base
+        del dev, weights
+        torch.cuda.empty_cache()
+
+    out = {
+        "metric": "moe_layer_tokens_per_s",
+        "value": headline["tokens_per_s"],
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": headline["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.shape} INT8 W8A8 MoE layer, M={args.m} tokens per step, top-8 of 128 experts, "
+                        f"H=2048 I=768, moe_align block 64, {args.weight_copies} rotating weight copies",
+            "shape": args.shape,
+            "tokens_per_step": args.m,
+            "gemm_variant": args.variant,
+        },
+        "roofline": {k: headline["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")},
+        "roofline_kernel": headline["roofline"]["kernel"],
+        "roofline_kernel_us": headline["roofline"]["kernel_us"],
+        "layer_int8_tops": headline["layer_int8_tops"],
+        "layer_mfma_frac": headline["layer_mfma_frac"],
+        "layer_hbm_gbps": headline["layer_hbm_gbps"],
+        "layer_hbm_frac": headline["layer_hbm_frac"],
+        "sweep": sweep,
+    }
+    if not args.no_cpu:
+        oracle = importlib.import_module("oracle.moe_i8_oracle")
+        out["cpu_baseline"] = cpu_baseline(oracle, torch, base_headline, args.cpu_sample)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

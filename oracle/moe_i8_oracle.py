@@ -75,7 +75,9 @@ def per_token_quant_int8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
         (*xf.shape[:-1], 1), 1e-10
     )
     scale = absmax / 127.0
-    inv = 127.0 / absmax
+    # tensor / tensor is one correctly rounded IEEE division; `127.0 / absmax` on a torch tensor is
+    # evaluated as reciprocal-then-multiply (two roundings) and flips near-tie elements.
+    inv = torch.full_like(absmax, 127.0) / absmax
     q = round_half_away(xf * inv).to(torch.int8)
     return q, scale
 
