@@ -23,6 +23,7 @@ HIPCC_FLAGS = [
     "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    "-Wno-inline-asm",
 ]
 
 
