@@ -28,11 +28,44 @@ __device__ __forceinline__ float round_to_bf16(float f) {
   return bf16_bits_to_f32(f32_to_bf16_bits(f));
 }
 
-// SiLU-gated product with the rounding points of a bf16 silu_and_mul kernel:
-// silu in fp32, rounded to bf16, times up in fp32, rounded to bf16.
-__device__ __forceinline__ uint32_t silu_mul_bf16_bits(float gate, float up) {
-  float s = round_to_bf16(gate / (1.0f + expf(-gate)));
-  return f32_to_bf16_bits(s * up);
+typedef float f2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+
+// Two fp32 -> packed bf16 (v_cvt_pk_bf16_f32, round to nearest even); lo in bits 15:0.
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  const bf2 b = __builtin_convertvector(f2{lo, hi}, bf2);
+  return *reinterpret_cast<const uint32_t*>(&b);
+}
+
+// SiLU with the hardware exp2 / reciprocal approximations (a few fp32 ulp); every GEMM family uses
+// this one definition so that the result does not depend on which kernel ran.
+__device__ __forceinline__ float fast_silu(float g) {
+  return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g));
+}
+
+// Four (gate, up) accumulator pairs -> four bf16 outputs with the rounding points of an unfused
+// pipeline: gate and up rounded to bf16, silu(gate) rounded to bf16, product rounded to bf16.
+__device__ __forceinline__ uint2 silu_mul_epilogue4(const int (&g)[4], const int (&u)[4], float a_scale,
+                                                    const float4& wg, const float4& wu) {
+  const float wgv[4] = {wg.x, wg.y, wg.z, wg.w};
+  const float wuv[4] = {wu.x, wu.y, wu.z, wu.w};
+  float h[4];
+#pragma unroll
+  for (int r = 0; r < 4; r += 2) {
+    const uint32_t g2 = pack_bf16((float)g[r] * a_scale * wgv[r], (float)g[r + 1] * a_scale * wgv[r + 1]);
+    const uint32_t u2 = pack_bf16((float)u[r] * a_scale * wuv[r], (float)u[r + 1] * a_scale * wuv[r + 1]);
+    const uint32_t s2 =
+        pack_bf16(fast_silu(__uint_as_float(g2 << 16)), fast_silu(__uint_as_float(g2 & 0xffff0000u)));
+    h[r] = __uint_as_float(s2 << 16) * __uint_as_float(u2 << 16);
+    h[r + 1] = __uint_as_float(s2 & 0xffff0000u) * __uint_as_float(u2 & 0xffff0000u);
+  }
+  return make_uint2(pack_bf16(h[0], h[1]), pack_bf16(h[2], h[3]));
+}
+
+// Four down-projection accumulators -> four bf16 outputs: acc * a_scale * w_scale * routed weight.
+__device__ __forceinline__ uint2 down_epilogue4(const int (&acc)[4], float a_scale, const float4& ws, float rw) {
+  return make_uint2(pack_bf16((float)acc[0] * a_scale * ws.x * rw, (float)acc[1] * a_scale * ws.y * rw),
+                    pack_bf16((float)acc[2] * a_scale * ws.z * rw, (float)acc[3] * a_scale * ws.w * rw));
 }
 
 // ---- launchers (defined one per .hip file; all asynchronous on `stream`) ----

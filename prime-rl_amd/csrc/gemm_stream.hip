@@ -131,13 +131,8 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
         if (!wok[t]) continue;
         const int n = wrow[t] + 4 * grp;
         const float4 ws = *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + n);
-        const float wsv[4] = {ws.x, ws.y, ws.z, ws.w};
-        uint32_t b[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          b[r] = f32_to_bf16_bits((float)acc[t][s][r] * as * wsv[r] * rw);
-        *reinterpret_cast<uint2*>(out + (int64_t)tok[s] * p.N + n) =
-            make_uint2(b[0] | (b[1] << 16), b[2] | (b[3] << 16));
+        const int v[4] = {acc[t][s][0], acc[t][s][1], acc[t][s][2], acc[t][s][3]};
+        *reinterpret_cast<uint2*>(out + (int64_t)tok[s] * p.N + n) = down_epilogue4(v, as, ws, rw);
       }
     }
   } else {  // kGateUpSilu: tiles come in (gate, up) pairs; out is [P, N / 2]
@@ -154,17 +149,9 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
         const float4 wg = *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + n);
         const float4 wu =
             *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + inter + n);
-        const float wgv[4] = {wg.x, wg.y, wg.z, wg.w};
-        const float wuv[4] = {wu.x, wu.y, wu.z, wu.w};
-        uint32_t b[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float g = round_to_bf16((float)acc[t][s][r] * as * wgv[r]);
-          const float u = round_to_bf16((float)acc[t + 1][s][r] * as * wuv[r]);
-          b[r] = silu_mul_bf16_bits(g, u);
-        }
-        *reinterpret_cast<uint2*>(out + (int64_t)tok[s] * inter + n) =
-            make_uint2(b[0] | (b[1] << 16), b[2] | (b[3] << 16));
+        const int g[4] = {acc[t][s][0], acc[t][s][1], acc[t][s][2], acc[t][s][3]};
+        const int u[4] = {acc[t + 1][s][0], acc[t + 1][s][1], acc[t + 1][s][2], acc[t + 1][s][3]};
+        *reinterpret_cast<uint2*>(out + (int64_t)tok[s] * inter + n) = silu_mul_epilogue4(g, u, as, wg, wu);
       }
     }
   }

@@ -1,6 +1,6 @@
 """GPU parity for the grouped int8 GEMMs through the C-ABI: int32 accumulators bit-exact, the down
-epilogue bit-exact, the SiLU-gated epilogue to within one bf16 step (the only difference is the
-last bit of expf)."""
+epilogue bit-exact, the SiLU-gated epilogue to within bf16 rounding noise (the only difference is
+the last bits of exp and of the reciprocal before two bf16 roundings)."""
 
 import pytest
 import torch
@@ -56,7 +56,8 @@ def test_int32_accumulators_bit_exact(pra, oracle, variant, E, k, H, I, M, B):
     acc1 = _skip_if_unsupported(pra, lambda: pra.gemm_acc_i32(
         st["x_q"].to(DEV), inp.w1.to(DEV), s, e, npp, k, B, P, variant))
     assert torch.equal(acc1.cpu(), st["acc1"]), int((acc1.cpu() != st["acc1"]).sum())
-    acc2 = pra.gemm_acc_i32(st["h_q"].to(DEV), inp.w2.to(DEV), s, e, npp, 1, B, P, variant)
+    acc2 = _skip_if_unsupported(pra, lambda: pra.gemm_acc_i32(
+        st["h_q"].to(DEV), inp.w2.to(DEV), s, e, npp, 1, B, P, variant))
     assert torch.equal(acc2.cpu(), st["acc2"]), int((acc2.cpu() != st["acc2"]).sum())
 
 
@@ -90,15 +91,18 @@ def test_down_gemm_epilogue_bit_exact(pra, oracle, variant, E, k, H, I, M, B):
 
 @pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("E,k,H,I,M,B", SHAPES)
-def test_gate_up_silu_within_one_bf16_step(pra, oracle, variant, E, k, H, I, M, B):
+def test_gate_up_silu_within_bf16_rounding(pra, oracle, variant, E, k, H, I, M, B):
     inp, st = _problem(oracle, E, k, H, I, M, seed=E + M + 2, B=B)
     s, e, npp = _routing_on_gpu(pra, inp, B)
     act = _skip_if_unsupported(pra, lambda: pra.gemm_gate_up_silu(
         st["x_q"].to(DEV), st["a1_scale"].to(DEV), inp.w1.to(DEV), inp.w1_scale.to(DEV), s, e, npp,
         k, B, M * k, variant))
+    # identical except where an fp32 value sits within a few ulp of a bf16 rounding boundary: then
+    # one bf16 step (two when the silu step is then doubled by the product's own rounding)
     d = bf16_ulp_diff(act, st["cache2"])
-    assert int(d.max()) <= 1, int(d.max())
-    assert float((d > 0).float().mean()) < 1e-3, float((d > 0).float().mean())
+    assert int(d.max()) <= 2, int(d.max())
+    assert float((d > 0).float().mean()) < 3e-3, float((d > 0).float().mean())
+    assert float((d > 1).float().mean()) < 2e-4, float((d > 1).float().mean())
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
