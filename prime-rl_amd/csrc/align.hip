@@ -17,8 +17,10 @@ constexpr int kSingleThreads = 1024;
 constexpr int kSingleWaves = kSingleThreads / kWave;
 constexpr int kMultiThreads = 256;
 constexpr int kMultiWaves = kMultiThreads / kWave;
-constexpr int kMultiChunk = 1024;         // pairs per wavefront in the multi-launch path
+constexpr int kMultiChunk = 1024;         // pairs per workgroup in the multi-launch path
 constexpr int64_t kSingleMaxPairs = 8192;  // above this the multi-launch path is used
+constexpr int kSingleIters = (int)(kSingleMaxPairs / kSingleWaves / kWave);  // 64-pair steps per wavefront
+constexpr int kMultiIters = kMultiChunk / kMultiWaves / kWave;
 
 // Lanes of this wavefront that are active and hold the same expert id as the caller.
 __device__ __forceinline__ uint64_t peers_of(int e, bool active, int nbits) {
@@ -31,13 +33,26 @@ __device__ __forceinline__ uint64_t peers_of(int e, bool active, int nbits) {
   return m;
 }
 
-// counts[e] += number of pairs in [begin, end) routed to e; counts is private to the wavefront.
-__device__ __forceinline__ void wave_histogram(const int32_t* __restrict__ ids, int64_t begin,
-                                               int64_t end, int E, int nbits, int* counts) {
+// Expert ids of the pairs [begin, end) this wavefront walks, 64 per iteration, all loads issued
+// before the first use (-1 past the end).
+template <int kIters>
+__device__ __forceinline__ void wave_load_ids(const int32_t* __restrict__ ids, int64_t begin, int64_t end,
+                                              int (&e)[kIters]) {
   const int lane = lane_id();
-  for (int64_t base = begin; base < end; base += kWave) {
-    const int64_t idx = base + lane;
-    int e = idx < end ? ids[idx] : -1;
+#pragma unroll
+  for (int i = 0; i < kIters; ++i) {
+    const int64_t idx = begin + i * kWave + lane;
+    e[i] = idx < end ? ids[idx] : -1;
+  }
+}
+
+// counts[x] += number of loaded pairs routed to x; counts is private to the wavefront.
+template <int kIters>
+__device__ __forceinline__ void wave_histogram(const int (&ids)[kIters], int E, int nbits, int* counts) {
+  const int lane = lane_id();
+#pragma unroll
+  for (int i = 0; i < kIters; ++i) {
+    const int e = ids[i];
     const bool active = e >= 0 && e < E;
     const uint64_t peers = peers_of(e, active, nbits);
     const int rank = __popcll(peers & ((1ull << lane) - 1ull));
@@ -46,14 +61,14 @@ __device__ __forceinline__ void wave_histogram(const int32_t* __restrict__ ids, 
   }
 }
 
-// sorted[cursor[e]++] = idx for the pairs in [begin, end), in ascending idx order per expert.
-__device__ __forceinline__ void wave_scatter(const int32_t* __restrict__ ids, int64_t begin,
-                                             int64_t end, int E, int nbits, int* cursor,
-                                             int32_t* __restrict__ sorted, int64_t sorted_cap) {
+// sorted[cursor[x]++] = pair index, in ascending pair index per expert.
+template <int kIters>
+__device__ __forceinline__ void wave_scatter(const int (&ids)[kIters], int64_t begin, int E, int nbits,
+                                             int* cursor, int32_t* __restrict__ sorted, int64_t sorted_cap) {
   const int lane = lane_id();
-  for (int64_t base = begin; base < end; base += kWave) {
-    const int64_t idx = base + lane;
-    int e = idx < end ? ids[idx] : -1;
+#pragma unroll
+  for (int i = 0; i < kIters; ++i) {
+    const int e = ids[i];
     const bool active = e >= 0 && e < E;
     const uint64_t peers = peers_of(e, active, nbits);
     const int rank = __popcll(peers & ((1ull << lane) - 1ull));
@@ -62,7 +77,7 @@ __device__ __forceinline__ void wave_scatter(const int32_t* __restrict__ ids, in
     __builtin_amdgcn_wave_barrier();
     if (active && rank == 0) cursor[e] += __popcll(peers);
     __builtin_amdgcn_wave_barrier();
-    if (active && pos < sorted_cap) sorted[pos] = (int32_t)idx;
+    if (active && pos < sorted_cap) sorted[pos] = (int32_t)(begin + i * kWave + lane);
   }
 }
 
@@ -133,7 +148,9 @@ __global__ __launch_bounds__(kSingleThreads) void align_single_kernel(
   const int per_wave = ((P + kSingleWaves - 1) / kSingleWaves + kWave - 1) / kWave * kWave;
   const int64_t begin = (int64_t)wave * per_wave < P ? (int64_t)wave * per_wave : P;
   const int64_t end = begin + per_wave < P ? begin + per_wave : P;
-  wave_histogram(ids, begin, end, E, nbits, hist + wave * E);
+  int mine[kSingleIters];
+  wave_load_ids(ids, begin, end, mine);
+  wave_histogram(mine, E, nbits, hist + wave * E);
   __syncthreads();
 
   int padded = 0;
@@ -158,39 +175,47 @@ __global__ __launch_bounds__(kSingleThreads) void align_single_kernel(
     for (int w = 0; w < kSingleWaves; ++w) hist[w * E + tid] += start;
   write_expert_ids(seg, E, B, npp, expert_ids, expert_cap);
   __syncthreads();
-  wave_scatter(ids, begin, end, E, nbits, hist + wave * E, sorted, sorted_cap);
+  wave_scatter(mine, begin, E, nbits, hist + wave * E, sorted, sorted_cap);
 }
 
 // ---- multi-launch path -------------------------------------------------------------------
-// workspace: unit_hist[units][E] | seg[E + 1]
+// One 256-thread workgroup per unit of kMultiChunk pairs; wavefront w of a unit walks the w-th
+// quarter.  workspace: unit_hist[units][E] | unit_base[units][E] | seg[E + 1]
+
+// smem[w][e] = number of pairs of wavefront w's quarter routed to e
+__device__ __forceinline__ void unit_wave_histograms(const int (&mine)[kMultiIters], int E, int nbits, int* smem) {
+  const int tid = threadIdx.x;
+  for (int i = tid; i < kMultiWaves * E; i += kMultiThreads) smem[i] = 0;
+  __syncthreads();
+  wave_histogram(mine, E, nbits, smem + (tid / kWave) * E);
+  __syncthreads();
+}
 
 __global__ __launch_bounds__(kMultiThreads) void align_hist_kernel(
-    const int32_t* __restrict__ ids, int64_t P, int E, int nbits, int units,
-    int32_t* __restrict__ unit_hist, int32_t* __restrict__ sorted, int64_t sorted_cap) {
+    const int32_t* __restrict__ ids, int64_t P, int E, int nbits, int32_t* __restrict__ unit_hist,
+    int32_t* __restrict__ sorted, int64_t sorted_cap) {
   extern __shared__ int smem[];
   const int tid = threadIdx.x;
-  const int wave = tid / kWave;
+  const int64_t begin = (int64_t)blockIdx.x * kMultiChunk + (tid / kWave) * (kMultiChunk / kMultiWaves);
+  const int64_t end = begin + kMultiChunk / kMultiWaves < P ? begin + kMultiChunk / kMultiWaves : P;
+  int mine[kMultiIters];
+  wave_load_ids(ids, begin, end, mine);
   for (int64_t i = (int64_t)blockIdx.x * kMultiThreads + tid; i < sorted_cap;
        i += (int64_t)gridDim.x * kMultiThreads)
     sorted[i] = (int32_t)P;
-  for (int i = tid; i < kMultiWaves * E; i += kMultiThreads) smem[i] = 0;
-  __syncthreads();
-  const int unit = blockIdx.x * kMultiWaves + wave;
-  if (unit < units) {
-    const int64_t begin = (int64_t)unit * kMultiChunk;
-    const int64_t end = begin + kMultiChunk < P ? begin + kMultiChunk : P;
-    wave_histogram(ids, begin, end, E, nbits, smem + wave * E);
-  }
-  __syncthreads();
-  for (int i = tid; i < kMultiWaves * E; i += kMultiThreads) {
-    const int u = blockIdx.x * kMultiWaves + i / E;
-    if (u < units) unit_hist[(int64_t)u * E + i % E] = smem[i];
+  unit_wave_histograms(mine, E, nbits, smem);
+  for (int e = tid; e < E; e += kMultiThreads) {
+    int sum = 0;
+#pragma unroll
+    for (int w = 0; w < kMultiWaves; ++w) sum += smem[w * E + e];
+    unit_hist[(int64_t)blockIdx.x * E + e] = sum;
   }
 }
 
 __global__ __launch_bounds__(kSingleThreads) void align_scan_kernel(
-    int E, int B, int units, int32_t* __restrict__ unit_hist, int32_t* __restrict__ seg_out,
-    int32_t* __restrict__ expert_ids, int64_t expert_cap, int32_t* __restrict__ npp_out) {
+    int E, int B, int units, const int32_t* __restrict__ unit_hist, int32_t* __restrict__ unit_base,
+    int32_t* __restrict__ seg_out, int32_t* __restrict__ expert_ids, int64_t expert_cap,
+    int32_t* __restrict__ npp_out) {
   __shared__ int seg[kMaxExperts + 1];
   __shared__ int wave_sums[kSingleWaves + 1];
   const int tid = threadIdx.x;
@@ -200,7 +225,7 @@ __global__ __launch_bounds__(kSingleThreads) void align_scan_kernel(
 #pragma unroll 8
     for (int u = 0; u < units; ++u) {
       const int c = unit_hist[(int64_t)u * E + tid];
-      unit_hist[(int64_t)u * E + tid] = run;
+      unit_base[(int64_t)u * E + tid] = run;
       run += c;
     }
     padded = (run + B - 1) / B * B;
@@ -221,24 +246,27 @@ __global__ __launch_bounds__(kSingleThreads) void align_scan_kernel(
 }
 
 __global__ __launch_bounds__(kMultiThreads) void align_scatter_kernel(
-    const int32_t* __restrict__ ids, int64_t P, int E, int nbits, int units,
-    const int32_t* __restrict__ unit_hist, const int32_t* __restrict__ seg,
-    int32_t* __restrict__ sorted, int64_t sorted_cap) {
+    const int32_t* __restrict__ ids, int64_t P, int E, int nbits, const int32_t* __restrict__ unit_base,
+    const int32_t* __restrict__ seg, int32_t* __restrict__ sorted, int64_t sorted_cap) {
   extern __shared__ int smem[];
   const int tid = threadIdx.x;
-  const int wave = tid / kWave;
-  for (int i = tid; i < kMultiWaves * E; i += kMultiThreads) {
-    const int u = blockIdx.x * kMultiWaves + i / E;
-    const int e = i % E;
-    smem[i] = u < units ? seg[e] + unit_hist[(int64_t)u * E + e] : 0;
+  const int64_t begin = (int64_t)blockIdx.x * kMultiChunk + (tid / kWave) * (kMultiChunk / kMultiWaves);
+  const int64_t end = begin + kMultiChunk / kMultiWaves < P ? begin + kMultiChunk / kMultiWaves : P;
+  int mine[kMultiIters];
+  wave_load_ids(ids, begin, end, mine);
+  unit_wave_histograms(mine, E, nbits, smem);
+  // counts -> write cursors: segment start + pairs of earlier units + pairs of earlier wavefronts
+  for (int e = tid; e < E; e += kMultiThreads) {
+    int run = seg[e] + unit_base[(int64_t)blockIdx.x * E + e];
+#pragma unroll
+    for (int w = 0; w < kMultiWaves; ++w) {
+      const int c = smem[w * E + e];
+      smem[w * E + e] = run;
+      run += c;
+    }
   }
   __syncthreads();
-  const int unit = blockIdx.x * kMultiWaves + wave;
-  if (unit < units) {
-    const int64_t begin = (int64_t)unit * kMultiChunk;
-    const int64_t end = begin + kMultiChunk < P ? begin + kMultiChunk : P;
-    wave_scatter(ids, begin, end, E, nbits, smem + wave * E, sorted, sorted_cap);
-  }
+  wave_scatter(mine, begin, E, nbits, smem + (tid / kWave) * E, sorted, sorted_cap);
 }
 
 int bits_for(int E) {
@@ -252,7 +280,7 @@ int bits_for(int E) {
 int64_t align_workspace_ints(int64_t num_pairs, int num_experts) {
   if (num_pairs <= kSingleMaxPairs) return 0;
   const int64_t units = (num_pairs + kMultiChunk - 1) / kMultiChunk;
-  return units * num_experts + num_experts + 1;
+  return 2 * units * num_experts + num_experts + 1;
 }
 
 hipError_t launch_align(const AlignArgs& a, hipStream_t stream) {
@@ -270,20 +298,21 @@ hipError_t launch_align(const AlignArgs& a, hipStream_t stream) {
     return hipGetLastError();
   }
   const int units = (int)((a.num_pairs + kMultiChunk - 1) / kMultiChunk);
-  const int blocks = (units + kMultiWaves - 1) / kMultiWaves;
   int32_t* unit_hist = a.workspace;
-  int32_t* seg = a.workspace + (int64_t)units * E;
+  int32_t* unit_base = unit_hist + (int64_t)units * E;
+  int32_t* seg = unit_base + (int64_t)units * E;
   const size_t lds = sizeof(int) * (size_t)kMultiWaves * E;
-  hipLaunchKernelGGL(align_hist_kernel, dim3(blocks), dim3(kMultiThreads), lds, stream, a.topk_ids,
-                     a.num_pairs, E, nbits, units, unit_hist, a.sorted_token_ids, a.sorted_cap);
+  hipLaunchKernelGGL(align_hist_kernel, dim3(units), dim3(kMultiThreads), lds, stream, a.topk_ids,
+                     a.num_pairs, E, nbits, unit_hist, a.sorted_token_ids, a.sorted_cap);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return err;
   hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kSingleThreads), 0, stream, E, a.block_size,
-                     units, unit_hist, seg, a.expert_ids, a.expert_cap, a.num_tokens_post_padded);
+                     units, unit_hist, unit_base, seg, a.expert_ids, a.expert_cap,
+                     a.num_tokens_post_padded);
   err = hipGetLastError();
   if (err != hipSuccess) return err;
-  hipLaunchKernelGGL(align_scatter_kernel, dim3(blocks), dim3(kMultiThreads), lds, stream,
-                     a.topk_ids, a.num_pairs, E, nbits, units, unit_hist, seg, a.sorted_token_ids,
+  hipLaunchKernelGGL(align_scatter_kernel, dim3(units), dim3(kMultiThreads), lds, stream,
+                     a.topk_ids, a.num_pairs, E, nbits, unit_base, seg, a.sorted_token_ids,
                      a.sorted_cap);
   return hipGetLastError();
 }

@@ -65,10 +65,16 @@ __device__ __forceinline__ void wait_vmcnt() {
 // 16 bytes per lane from global memory straight into LDS: lane i lands at lds_addr + 16 * i
 // (lds_addr is wave-uniform and goes through M0).  Issued as inline assembly so that the waits are
 // the explicit vmcnt waits of the ring below and not a conservative vmcnt(0) before every LDS read.
-__device__ __forceinline__ void load_to_lds_16(const int8_t* src, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+// The source is a wave-uniform base (SGPR pair) plus an unsigned 32-bit byte offset per lane.
+__device__ __forceinline__ void load_to_lds_16(const int8_t* base, uint32_t offset, uint32_t lds_addr) {
+  const uint64_t b = reinterpret_cast<uint64_t>(base);
+  // readfirstlane yields a signed int: go through uint32_t so that the low half is not sign-extended
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
+  const uint64_t ub = (uint64_t)lo | ((uint64_t)hi << 32);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
-               : "s"(lds_addr), "v"(src)
+               : "s"((uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(offset), "s"(ub)
                : "memory", "m0");
 }
 
@@ -153,8 +159,9 @@ struct Task {
 };
 
 struct TaskLoads {
-  const int8_t* wsrc[4];
-  const int8_t* xsrc[4];
+  const int8_t* wbase;  // weights of the task's expert (wave-uniform)
+  uint32_t woff[4];     // per lane: byte offset of its chunk of weight row i from wbase
+  uint32_t xoff[4];     // per lane: byte offset of its chunk of token row i from a_q
 };
 
 // Lane fills LDS slot (lane & 7) of row 32 * wave + 8 * i + (lane >> 3): it fetches the logical
@@ -175,24 +182,25 @@ __device__ __forceinline__ void setup_loads(const TileParams& p, const Task& tk,
       const int ch = tk.nt * kBN + row;
       n = ch < p.N ? ch : p.N - 1;
     }
-    ld.wsrc[i] = p.w + ((int64_t)tk.e * p.N + n) * K + chunk;
-    int64_t arow = 0;
+    ld.woff[i] = (uint32_t)n * (uint32_t)K + chunk;
+    uint32_t arow = 0;
     if ((wave >> 1) < tk.nsub) {
       const int32_t tok = p.sorted_ids[tk.slot0 + row];
-      if (tok >= 0 && tok < p.P) arow = tok / p.row_div;
+      if (tok >= 0 && tok < p.P) arow = (uint32_t)(tok / p.row_div);
     }
-    ld.xsrc[i] = p.a_q + arow * K + chunk;
+    ld.xoff[i] = arow * (uint32_t)K + chunk;
   }
+  ld.wbase = p.w + (int64_t)tk.e * p.N * K;
 }
 
-__device__ __forceinline__ void issue_stage_loads(const TaskLoads& ld, uint32_t stage_addr, int wave, int koff,
-                                                  bool tokens) {
+__device__ __forceinline__ void issue_stage_loads(const TaskLoads& ld, const int8_t* a_q, uint32_t stage_addr,
+                                                  int wave, int koff, bool tokens) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) load_to_lds_16(ld.wsrc[i] + koff, stage_addr + (wave * 4 + i) * 1024);
+  for (int i = 0; i < 4; ++i) load_to_lds_16(ld.wbase + koff, ld.woff[i], stage_addr + (wave * 4 + i) * 1024);
   if (tokens) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      load_to_lds_16(ld.xsrc[i] + koff, stage_addr + kTokOffset + (wave * 4 + i) * 1024);
+      load_to_lds_16(a_q + koff, ld.xoff[i], stage_addr + kTokOffset + (wave * 4 + i) * 1024);
   }
 }
 
@@ -228,19 +236,27 @@ __device__ __forceinline__ void multiply_stage(const TileReads& rd, const char* 
 }
 
 // acc[ci][tj][4q + r] is channel base(ci) + 8q + 4 * (lane >> 5) + r of token row
-// tb * 64 + tj * 32 + (lane & 31) of the tile.
+// tb * 64 + tj * 32 + (lane & 31) of the tile.  The bf16 results are transposed through an 8 KB
+// LDS region private to the wavefront so that the global stores are 16 bytes per lane and cover
+// whole cache lines of an output row (rows of 16-byte chunks, chunk index XOR-swizzled with the row
+// so that neither the 8-byte writes nor the 16-byte reads pile up on a bank).
 template <int MODE>
 __device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, int chh, int tb, int lane,
-                                         v16i (&acc)[4][2]) {
+                                         v16i (&acc)[4][2], char* wave_lds) {
   const int lrow = lane & 31;
   const int lhalf = lane >> 5;
   const int inter = p.N / 2;
+  int32_t tok[2];
 #pragma unroll
   for (int tj = 0; tj < 2; ++tj) {
-    const int32_t tok = p.sorted_ids[tk.slot0 + tb * 64 + tj * 32 + lrow];
-    if (tok < 0 || tok >= p.P) continue;
-    if constexpr (MODE == kAccI32) {
-      int32_t* out = static_cast<int32_t*>(p.out) + (int64_t)tok * p.N;
+    tok[tj] = p.sorted_ids[tk.slot0 + tb * 64 + tj * 32 + lrow];
+    if (tok[tj] < 0 || tok[tj] >= p.P) tok[tj] = -1;
+  }
+  if constexpr (MODE == kAccI32) {
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+      if (tok[tj] < 0) continue;
+      int32_t* out = static_cast<int32_t*>(p.out) + (int64_t)tok[tj] * p.N;
 #pragma unroll
       for (int ci = 0; ci < 4; ++ci)
 #pragma unroll
@@ -250,38 +266,70 @@ __device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, in
             *reinterpret_cast<v4i*>(out + n) =
                 v4i{acc[ci][tj][4 * q], acc[ci][tj][4 * q + 1], acc[ci][tj][4 * q + 2], acc[ci][tj][4 * q + 3]};
         }
-    } else if constexpr (MODE == kDown) {
-      uint16_t* out = static_cast<uint16_t*>(p.out) + (int64_t)tok * p.N;
-      const float as = p.a_scale[tok / p.row_div];
-      const float rw = p.row_weight[tok];
-      const float* wsc = p.w_scale + (int64_t)tk.e * p.N;
+    }
+  } else if constexpr (MODE == kDown) {
+    const float* wsc = p.w_scale + (int64_t)tk.e * p.N;
+    const int n0 = tk.nt * kBN + chh * 128;  // first channel of this wavefront
 #pragma unroll
-      for (int ci = 0; ci < 4; ++ci)
+    for (int tj = 0; tj < 2; ++tj) {
+      // 32 token rows x 128 channels: rows of 256 bytes = 16 chunks
+      const float as = tok[tj] >= 0 ? p.a_scale[tok[tj] / p.row_div] : 0.0f;
+      const float rw = tok[tj] >= 0 ? p.row_weight[tok[tj]] : 0.0f;
+#pragma unroll
+      for (int ci = 0; ci < 4; ++ci) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int n = tk.nt * kBN + chh * 128 + ci * 32 + 8 * q + 4 * lhalf;
-          if (n >= p.N) continue;
-          const float4 ws = *reinterpret_cast<const float4*>(wsc + n);
+          const int n = n0 + ci * 32 + 8 * q + 4 * lhalf;
+          const float4 ws = *reinterpret_cast<const float4*>(wsc + (n < p.N ? n : 0));
           const int v[4] = {acc[ci][tj][4 * q], acc[ci][tj][4 * q + 1], acc[ci][tj][4 * q + 2], acc[ci][tj][4 * q + 3]};
-          *reinterpret_cast<uint2*>(out + n) = down_epilogue4(v, as, ws, rw);
+          *reinterpret_cast<uint2*>(wave_lds + lrow * 256 + (((ci * 4 + q) ^ (lrow & 15)) * 16) + lhalf * 8) =
+              down_epilogue4(v, as, ws, rw);
         }
-    } else {
-      uint16_t* out = static_cast<uint16_t*>(p.out) + (int64_t)tok * inter;
-      const float as = p.a_scale[tok / p.row_div];
-      const float* wsc = p.w_scale + (int64_t)tk.e * p.N;
+        __builtin_amdgcn_sched_barrier(0);  // keep the scale loads of later groups from piling up in VGPRs
+      }
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const int row = r * 4 + (lane >> 4);
+        const int chunk = lane & 15;
+        const uint4 v = *reinterpret_cast<const uint4*>(wave_lds + row * 256 + ((chunk ^ (row & 15)) * 16));
+        const int32_t t = __shfl(tok[tj], row);
+        const int n = n0 + chunk * 8;
+        if (t >= 0 && n < p.N)
+          *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.out) + (int64_t)t * p.N + n) = v;
+      }
+    }
+  } else {
+    const float* wsc = p.w_scale + (int64_t)tk.e * p.N;
+    const int n0 = tk.nt * 128 + chh * 64;  // first gate channel of this wavefront
+    // 64 token rows x 64 channels: rows of 128 bytes = 8 chunks
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+      const float as = tok[tj] >= 0 ? p.a_scale[tok[tj] / p.row_div] : 0.0f;
+      const int row = tj * 32 + lrow;
 #pragma unroll
       for (int ci = 0; ci < 2; ++ci)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int n = tk.nt * 128 + chh * 64 + ci * 32 + 8 * q + 4 * lhalf;  // gate channel
-          if (n >= inter) continue;
-          const float4 wg = *reinterpret_cast<const float4*>(wsc + n);
-          const float4 wu = *reinterpret_cast<const float4*>(wsc + inter + n);
+          const int n = n0 + ci * 32 + 8 * q + 4 * lhalf;
+          const int ns = n < inter ? n : 0;
+          const float4 wg = *reinterpret_cast<const float4*>(wsc + ns);
+          const float4 wu = *reinterpret_cast<const float4*>(wsc + inter + ns);
           const int g[4] = {acc[ci][tj][4 * q], acc[ci][tj][4 * q + 1], acc[ci][tj][4 * q + 2], acc[ci][tj][4 * q + 3]};
           const int u[4] = {acc[ci + 2][tj][4 * q], acc[ci + 2][tj][4 * q + 1], acc[ci + 2][tj][4 * q + 2],
                             acc[ci + 2][tj][4 * q + 3]};
-          *reinterpret_cast<uint2*>(out + n) = silu_mul_epilogue4(g, u, as, wg, wu);
+          *reinterpret_cast<uint2*>(wave_lds + row * 128 + (((ci * 4 + q) ^ (row & 7)) * 16) + lhalf * 8) =
+              silu_mul_epilogue4(g, u, as, wg, wu);
         }
+    }
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int row = r * 8 + (lane >> 3);
+      const int chunk = lane & 7;
+      const uint4 v = *reinterpret_cast<const uint4*>(wave_lds + row * 128 + ((chunk ^ (row & 7)) * 16));
+      const int32_t t = __shfl(tok[r >> 2], row & 31);
+      const int n = n0 + chunk * 8;
+      if (t >= 0 && n < inter)
+        *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.out) + (int64_t)t * inter + n) = v;
     }
   }
 }
@@ -360,7 +408,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(TileParams p) {
   int parity = 0;
   // The scratch of the tile list lived in the stage memory; everybody is past it (the builder ends
   // with a barrier), so the first stage can be filled now.
-  issue_stage_loads(ld, stage0, wave, 0, my_tokens);
+  issue_stage_loads(ld, p.a_q, stage0, wave, 0, my_tokens);
 
   while (true) {
     v16i acc[4][2];
@@ -386,13 +434,16 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(TileParams p) {
       __builtin_amdgcn_s_barrier();
       const uint32_t other = stage0 + (parity ^ 1) * kStageBytes;
       if (s + 1 < nk)
-        issue_stage_loads(ld, other, wave, (s + 1) * kBK, my_tokens);
+        issue_stage_loads(ld, p.a_q, other, wave, (s + 1) * kBK, my_tokens);
       else if (nx.e >= 0)
-        issue_stage_loads(nld, other, wave, 0, nx_tokens);
+        issue_stage_loads(nld, p.a_q, other, wave, 0, nx_tokens);
       if (my_tokens) multiply_stage(rd, stages + parity * kStageBytes, acc);
       parity ^= 1;
     }
-    if (my_tokens) epilogue<MODE>(p, tk, chh, tb, lane, acc);
+    // everybody is done reading the stage of the last step: it becomes the epilogue's staging area
+    // (the next task's first loads went to the other stage)
+    __builtin_amdgcn_s_barrier();
+    if (my_tokens) epilogue<MODE>(p, tk, chh, tb, lane, acc, stages + (parity ^ 1) * kStageBytes + wave * 8192);
     if (nx.e < 0) break;
     tk = nx;
     ld = nld;
@@ -439,8 +490,12 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
 }  // namespace
 
 bool gemm_tile_supports(const GemmArgs& a) {
+  // per-lane source offsets are 32-bit: one expert's weights and the activation matrix must each
+  // span less than 4 GiB
+  const int64_t act_rows = (a.num_pairs + a.row_div - 1) / a.row_div;
   return (a.block_size == 64 || a.block_size == 128) && a.k % kBK == 0 && a.k >= 2 * kBK && a.n % 16 == 0 &&
-         (a.sorted_cap + a.block_size - 1) / a.block_size <= kMaxTiles;
+         (a.sorted_cap + a.block_size - 1) / a.block_size <= kMaxTiles && (int64_t)a.n * a.k < (1ll << 32) &&
+         act_rows * a.k < (1ll << 32);
 }
 
 hipError_t launch_gemm_tile(const GemmArgs& a, hipStream_t stream) {

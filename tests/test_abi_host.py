@@ -36,7 +36,7 @@ def test_capacity_and_workspace_formulas(pra):
     assert lib.moe_i8_sorted_capacity(0, 8, 64) == 0
     assert lib.moe_i8_align_workspace_bytes(1024, 128, 64) == 0
     big = lib.moe_i8_align_workspace_bytes(131072, 256, 64)
-    assert big == 4 * (128 * 256 + 257)
+    assert big == 4 * (2 * 128 * 256 + 257)
     ws = lib.moe_i8_workspace_bytes(16, 8, 128, 2048, 768, 64)
     P = 128
     assert ws >= 16 * 2048 + P * 768 * 3 + P * 2048 * 2 and ws % 256 == 0
