@@ -48,10 +48,12 @@ __device__ __forceinline__ void wave_load_ids(const int32_t* __restrict__ ids, i
 
 // counts[x] += number of loaded pairs routed to x; counts is private to the wavefront.
 template <int kIters>
-__device__ __forceinline__ void wave_histogram(const int (&ids)[kIters], int E, int nbits, int* counts) {
+__device__ __forceinline__ void wave_histogram(const int (&ids)[kIters], int64_t count, int E, int nbits,
+                                               int* counts) {
   const int lane = lane_id();
 #pragma unroll
   for (int i = 0; i < kIters; ++i) {
+    if ((int64_t)i * kWave >= count) break;  // wave-uniform: nothing left in this wavefront's range
     const int e = ids[i];
     const bool active = e >= 0 && e < E;
     const uint64_t peers = peers_of(e, active, nbits);
@@ -63,11 +65,13 @@ __device__ __forceinline__ void wave_histogram(const int (&ids)[kIters], int E, 
 
 // sorted[cursor[x]++] = pair index, in ascending pair index per expert.
 template <int kIters>
-__device__ __forceinline__ void wave_scatter(const int (&ids)[kIters], int64_t begin, int E, int nbits,
-                                             int* cursor, int32_t* __restrict__ sorted, int64_t sorted_cap) {
+__device__ __forceinline__ void wave_scatter(const int (&ids)[kIters], int64_t begin, int64_t count, int E,
+                                             int nbits, int* cursor, int32_t* __restrict__ sorted,
+                                             int64_t sorted_cap) {
   const int lane = lane_id();
 #pragma unroll
   for (int i = 0; i < kIters; ++i) {
+    if ((int64_t)i * kWave >= count) break;
     const int e = ids[i];
     const bool active = e >= 0 && e < E;
     const uint64_t peers = peers_of(e, active, nbits);
@@ -150,7 +154,7 @@ __global__ __launch_bounds__(kSingleThreads) void align_single_kernel(
   const int64_t end = begin + per_wave < P ? begin + per_wave : P;
   int mine[kSingleIters];
   wave_load_ids(ids, begin, end, mine);
-  wave_histogram(mine, E, nbits, hist + wave * E);
+  wave_histogram(mine, end - begin, E, nbits, hist + wave * E);
   __syncthreads();
 
   int padded = 0;
@@ -175,7 +179,7 @@ __global__ __launch_bounds__(kSingleThreads) void align_single_kernel(
     for (int w = 0; w < kSingleWaves; ++w) hist[w * E + tid] += start;
   write_expert_ids(seg, E, B, npp, expert_ids, expert_cap);
   __syncthreads();
-  wave_scatter(mine, begin, E, nbits, hist + wave * E, sorted, sorted_cap);
+  wave_scatter(mine, begin, end - begin, E, nbits, hist + wave * E, sorted, sorted_cap);
 }
 
 // ---- multi-launch path -------------------------------------------------------------------
@@ -183,11 +187,12 @@ __global__ __launch_bounds__(kSingleThreads) void align_single_kernel(
 // quarter.  workspace: unit_hist[units][E] | unit_base[units][E] | seg[E + 1]
 
 // smem[w][e] = number of pairs of wavefront w's quarter routed to e
-__device__ __forceinline__ void unit_wave_histograms(const int (&mine)[kMultiIters], int E, int nbits, int* smem) {
+__device__ __forceinline__ void unit_wave_histograms(const int (&mine)[kMultiIters], int64_t count, int E,
+                                                     int nbits, int* smem) {
   const int tid = threadIdx.x;
   for (int i = tid; i < kMultiWaves * E; i += kMultiThreads) smem[i] = 0;
   __syncthreads();
-  wave_histogram(mine, E, nbits, smem + (tid / kWave) * E);
+  wave_histogram(mine, count, E, nbits, smem + (tid / kWave) * E);
   __syncthreads();
 }
 
@@ -203,7 +208,7 @@ __global__ __launch_bounds__(kMultiThreads) void align_hist_kernel(
   for (int64_t i = (int64_t)blockIdx.x * kMultiThreads + tid; i < sorted_cap;
        i += (int64_t)gridDim.x * kMultiThreads)
     sorted[i] = (int32_t)P;
-  unit_wave_histograms(mine, E, nbits, smem);
+  unit_wave_histograms(mine, end - begin, E, nbits, smem);
   for (int e = tid; e < E; e += kMultiThreads) {
     int sum = 0;
 #pragma unroll
@@ -254,7 +259,7 @@ __global__ __launch_bounds__(kMultiThreads) void align_scatter_kernel(
   const int64_t end = begin + kMultiChunk / kMultiWaves < P ? begin + kMultiChunk / kMultiWaves : P;
   int mine[kMultiIters];
   wave_load_ids(ids, begin, end, mine);
-  unit_wave_histograms(mine, E, nbits, smem);
+  unit_wave_histograms(mine, end - begin, E, nbits, smem);
   // counts -> write cursors: segment start + pairs of earlier units + pairs of earlier wavefronts
   for (int e = tid; e < E; e += kMultiThreads) {
     int run = seg[e] + unit_base[(int64_t)blockIdx.x * E + e];
@@ -266,7 +271,7 @@ __global__ __launch_bounds__(kMultiThreads) void align_scatter_kernel(
     }
   }
   __syncthreads();
-  wave_scatter(mine, begin, E, nbits, smem + (tid / kWave) * E, sorted, sorted_cap);
+  wave_scatter(mine, begin, end - begin, E, nbits, smem + (tid / kWave) * E, sorted, sorted_cap);
 }
 
 int bits_for(int E) {

@@ -23,7 +23,16 @@ constexpr int kWaves = kThreads / kWave;
 constexpr int kSub = 16;    // token rows per sub-tile (MFMA N)
 constexpr int kGroup = 4;   // sub-tiles processed per pass over the weights
 constexpr int kStepK = 64;  // reduction bytes per MFMA
-constexpr int kUnroll = 4;  // MFMA steps whose loads are issued together
+#ifndef MOE_I8_STREAM_UNROLL
+#define MOE_I8_STREAM_UNROLL 4
+#endif
+#ifndef MOE_I8_STREAM_TPW
+#define MOE_I8_STREAM_TPW 2
+#endif
+#ifndef MOE_I8_STREAM_NT
+#define MOE_I8_STREAM_NT 1
+#endif
+constexpr int kUnroll = MOE_I8_STREAM_UNROLL;  // MFMA steps whose loads are issued together
 
 struct StreamParams {
   const int8_t* a_q;
@@ -42,6 +51,14 @@ struct StreamParams {
   int B;
   void* out;
 };
+
+__device__ __forceinline__ v4i load_weights(const int8_t* p) {
+#if MOE_I8_STREAM_NT
+  return __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
+#else
+  return *reinterpret_cast<const v4i*>(p);
+#endif
+}
 
 template <int MODE, int TPW, int NS>
 __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int e, int sub0,
@@ -80,8 +97,7 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
     for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
       for (int t = 0; t < TPW; ++t)
-        wv[u][t] = __builtin_nontemporal_load(
-            reinterpret_cast<const v4i*>(wp[t] + k0 + u * kStepK));
+        wv[u][t] = load_weights(wp[t] + k0 + u * kStepK);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
@@ -100,7 +116,7 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
     v4i av[NS];
 #pragma unroll
     for (int t = 0; t < TPW; ++t)
-      wv[t] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wp[t] + k0));
+      wv[t] = load_weights(wp[t] + k0);
 #pragma unroll
     for (int s = 0; s < NS; ++s) av[s] = *reinterpret_cast<const v4i*>(ap[s] + k0);
 #pragma unroll
@@ -241,9 +257,9 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
 
 hipError_t launch_gemm_stream(const GemmArgs& a, hipStream_t stream) {
   switch (a.mode) {
-    case kGateUpSilu: return launch_mode<kGateUpSilu, 2>(a, stream);
-    case kDown: return launch_mode<kDown, 2>(a, stream);
-    case kAccI32: return launch_mode<kAccI32, 2>(a, stream);
+    case kGateUpSilu: return launch_mode<kGateUpSilu, MOE_I8_STREAM_TPW>(a, stream);
+    case kDown: return launch_mode<kDown, MOE_I8_STREAM_TPW>(a, stream);
+    case kAccI32: return launch_mode<kAccI32, MOE_I8_STREAM_TPW>(a, stream);
     default: return hipErrorInvalidValue;
   }
 }
