@@ -1,8 +1,15 @@
 // Grouped int8 GEMM for gfx950, weight-streaming family (few rows per expert: decode).
 //
-// In this regime every weight byte is used by one 64-row block only, so the kernel is a pure
-// HBM stream: weights go global -> registers in the MFMA operand layout with 16-byte loads, never
-// through LDS, and the activation rows (a few KB per block) are re-read from the vector cache.
+// In this regime every weight byte is used by one 64-row block only, so the kernel is a pure HBM
+// stream and what matters is that DRAM sees long contiguous reads with many of them in flight.
+// Each wavefront owns 32 weight rows (two 16-row MFMA tiles; for the gate_up GEMM 16 gate rows and
+// the 16 matching up rows) and walks the reduction dimension in windows of 256 bytes per row.  A
+// window is fetched with eight 16-byte-per-lane loads, each covering 4 rows x 256 contiguous bytes,
+// and the loads of the next window are issued before the current one is consumed.  The registers
+// are then transposed into the MFMA operand layout through an 8 KB LDS area private to the
+// wavefront (16-byte chunks XOR-swizzled with the row, so that neither the row-linear writes nor
+// the 16-rows-same-chunk reads collide on a bank); no barrier is ever needed.  The few activation
+// rows of the block are read from global memory (vector cache) directly in the operand layout.
 //
 // v_mfma_i32_16x16x64_i8 is used "transposed": the A operand carries 16 weight rows (output
 // channels), the B operand 16 token rows, so each lane ends up with 4 consecutive channels of one
@@ -10,9 +17,9 @@
 // row/column l % 16 and the 16 reduction bytes [16 * (l / 16), +16) of each 64-byte step; both
 // operands use the same split, so the reduction order inside the instruction is immaterial.
 //
-// A 64-row block is handled as up to four 16-row sub-tiles; sub-tiles that hold only padding are
-// skipped (valid rows are a prefix of the block), so a block with 1..16 routed rows costs one
-// MFMA per 64 weight bytes per lane group.
+// A 64-row block is handled as 16-row sub-tiles, one pass over the weights each (a second pass
+// finds them in L2); sub-tiles that hold only padding are skipped (valid rows are a prefix of the
+// block).  Blocks with many rows belong to the LDS-tiled family.
 #include "common.hpp"
 
 namespace moe_i8 {
@@ -20,19 +27,14 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
-constexpr int kSub = 16;    // token rows per sub-tile (MFMA N)
-constexpr int kGroup = 4;   // sub-tiles processed per pass over the weights
-constexpr int kStepK = 64;  // reduction bytes per MFMA
-#ifndef MOE_I8_STREAM_UNROLL
-#define MOE_I8_STREAM_UNROLL 4
-#endif
-#ifndef MOE_I8_STREAM_TPW
-#define MOE_I8_STREAM_TPW 2
-#endif
-#ifndef MOE_I8_STREAM_NT
-#define MOE_I8_STREAM_NT 1
-#endif
-constexpr int kUnroll = MOE_I8_STREAM_UNROLL;  // MFMA steps whose loads are issued together
+constexpr int kSub = 16;      // token rows per sub-tile (MFMA N)
+constexpr int kGroup = 1;     // sub-tiles processed per pass over the weights
+constexpr int kStepK = 64;    // reduction bytes per MFMA
+constexpr int kTiles = 2;     // 16-row weight tiles per wavefront
+constexpr int kWinBytes = 256;                              // bytes of every weight row per window
+constexpr int kWinSteps = kWinBytes / kStepK;               // MFMA steps per window
+constexpr int kWinLoads = kTiles * 16 * kWinBytes / 1024;   // 1 KB wave-level loads per window
+constexpr int kWaveLds = kTiles * 16 * kWinBytes;           // LDS bytes per wavefront
 
 struct StreamParams {
   const int8_t* a_q;
@@ -52,17 +54,16 @@ struct StreamParams {
   void* out;
 };
 
-__device__ __forceinline__ v4i load_weights(const int8_t* p) {
-#if MOE_I8_STREAM_NT
-  return __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
-#else
-  return *reinterpret_cast<const v4i*>(p);
-#endif
-}
+template <int NS>
+struct Window {
+  v4i w[kWinLoads];
+  v4i a[NS][kWinSteps];
+};
 
-template <int MODE, int TPW, int NS>
+template <int MODE, int NS>
 __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int e, int sub0,
-                                            const int (&wrow)[TPW], const bool (&wok)[TPW]) {
+                                            const int (&wrow)[kTiles], const bool (&wok)[kTiles],
+                                            char* wave_lds) {
   const int lane = lane_id();
   const int col = lane & 15;  // token slot inside a sub-tile / weight row inside a tile
   const int grp = lane >> 4;  // which 16 reduction bytes of each step; which 4 output channels
@@ -78,59 +79,70 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
     const int64_t arow = tok_ok[s] ? tok[s] / p.row_div : 0;
     ap[s] = p.a_q + arow * K + grp * 16;
   }
-  const int8_t* wp[TPW];
+  // Load j of a window covers rows 4 * (j % 4) + (lane >> 4) of tile j / 4, chunk lane & 15.
+  const int ld_row = lane >> 4;
+  const int ld_chunk = lane & 15;
+  const int8_t* wp[kTiles];
 #pragma unroll
-  for (int t = 0; t < TPW; ++t)
-    wp[t] = p.w + ((int64_t)e * p.N + wrow[t] + col) * K + grp * 16;
+  for (int t = 0; t < kTiles; ++t)
+    wp[t] = p.w + ((int64_t)e * p.N + wrow[t] + ld_row) * K + ld_chunk * 16;
+  // LDS: [32 rows][256 B]; chunk c of row r sits at position c ^ (r & 15)
+  const int st_base = ld_row * kWinBytes + ((ld_chunk ^ ld_row) * 16);  // ^ (j % 4) * 64, + j * 1024
+  const int rd_base = col * kWinBytes + ((grp ^ col) * 16);             // ^ u * 64, + t * 4096
 
-  v4i acc[TPW][NS];
+  v4i acc[kTiles][NS];
 #pragma unroll
-  for (int t = 0; t < TPW; ++t)
+  for (int t = 0; t < kTiles; ++t)
 #pragma unroll
     for (int s = 0; s < NS; ++s) acc[t][s] = v4i{0, 0, 0, 0};
 
-  int k0 = 0;
-  for (; k0 + kStepK * kUnroll <= K; k0 += kStepK * kUnroll) {
-    v4i wv[kUnroll][TPW];
-    v4i av[kUnroll][NS];
+  auto fetch = [&](Window<NS>& win, int k0) {
+    const bool chunk_in = k0 + ld_chunk * 16 < K;  // only the last window of a ragged K is partial
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
+    for (int j = 0; j < kWinLoads; ++j) {
+      const int8_t* src = wp[j / 4] + (int64_t)(4 * (j % 4)) * K + k0;
+      win.w[j] = chunk_in ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src)) : v4i{0, 0, 0, 0};
+    }
 #pragma unroll
-      for (int t = 0; t < TPW; ++t)
-        wv[u][t] = load_weights(wp[t] + k0 + u * kStepK);
+    for (int s = 0; s < NS; ++s)
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
+      for (int u = 0; u < kWinSteps; ++u)
+        win.a[s][u] = k0 + u * kStepK < K ? *reinterpret_cast<const v4i*>(ap[s] + k0 + u * kStepK)
+                                           : v4i{0, 0, 0, 0};
+  };
+  auto consume = [&](const Window<NS>& win) {
 #pragma unroll
-      for (int s = 0; s < NS; ++s)
-        av[u][s] = *reinterpret_cast<const v4i*>(ap[s] + k0 + u * kStepK);
+    for (int j = 0; j < kWinLoads; ++j)
+      *reinterpret_cast<v4i*>(wave_lds + j * 1024 + (st_base ^ ((j % 4) * 64))) = win.w[j];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
+    for (int u = 0; u < kWinSteps; ++u) {
+      v4i frag[kTiles];
 #pragma unroll
-      for (int t = 0; t < TPW; ++t)
+      for (int t = 0; t < kTiles; ++t)
+        frag[t] = *reinterpret_cast<const v4i*>(wave_lds + t * 4096 + (rd_base ^ (u * 64)));
+#pragma unroll
+      for (int t = 0; t < kTiles; ++t)
 #pragma unroll
         for (int s = 0; s < NS; ++s)
-          acc[t][s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[u][t], av[u][s], acc[t][s], 0, 0, 0);
-  }
-  for (; k0 < K; k0 += kStepK) {
-    v4i wv[TPW];
-    v4i av[NS];
-#pragma unroll
-    for (int t = 0; t < TPW; ++t)
-      wv[t] = load_weights(wp[t] + k0);
-#pragma unroll
-    for (int s = 0; s < NS; ++s) av[s] = *reinterpret_cast<const v4i*>(ap[s] + k0);
-#pragma unroll
-    for (int t = 0; t < TPW; ++t)
-#pragma unroll
-      for (int s = 0; s < NS; ++s)
-        acc[t][s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[t], av[s], acc[t][s], 0, 0, 0);
+          acc[t][s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(frag[t], win.a[s][u], acc[t][s], 0, 0, 0);
+    }
+  };
+
+  Window<NS> w0, w1;
+  fetch(w0, 0);
+  for (int k0 = 0; k0 < K; k0 += 2 * kWinBytes) {
+    if (k0 + kWinBytes < K) fetch(w1, k0 + kWinBytes);
+    consume(w0);
+    if (k0 + kWinBytes >= K) break;
+    if (k0 + 2 * kWinBytes < K) fetch(w0, k0 + 2 * kWinBytes);
+    consume(w1);
   }
 
   // Epilogue: lane holds channels wrow[t] + 4 * grp + {0..3} of token tok[s].
   if constexpr (MODE == kAccI32) {
     int32_t* out = static_cast<int32_t*>(p.out);
 #pragma unroll
-    for (int t = 0; t < TPW; ++t)
+    for (int t = 0; t < kTiles; ++t)
 #pragma unroll
       for (int s = 0; s < NS; ++s)
         if (wok[t] && tok_ok[s])
@@ -143,7 +155,7 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
       const float as = p.a_scale[tok[s] / p.row_div];
       const float rw = p.row_weight[tok[s]];
 #pragma unroll
-      for (int t = 0; t < TPW; ++t) {
+      for (int t = 0; t < kTiles; ++t) {
         if (!wok[t]) continue;
         const int n = wrow[t] + 4 * grp;
         const float4 ws = *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + n);
@@ -151,31 +163,28 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
         *reinterpret_cast<uint2*>(out + (int64_t)tok[s] * p.N + n) = down_epilogue4(v, as, ws, rw);
       }
     }
-  } else {  // kGateUpSilu: tiles come in (gate, up) pairs; out is [P, N / 2]
+  } else {  // kGateUpSilu: tile 0 is gate, tile 1 the matching up rows; out is [P, N / 2]
     uint16_t* out = static_cast<uint16_t*>(p.out);
     const int inter = p.N / 2;
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-      if (!tok_ok[s]) continue;
+      if (!tok_ok[s] || !wok[0]) continue;
       const float as = p.a_scale[tok[s] / p.row_div];
-#pragma unroll
-      for (int t = 0; t < TPW; t += 2) {
-        if (!wok[t]) continue;
-        const int n = wrow[t] + 4 * grp;  // gate channel; up channel is n + inter
-        const float4 wg = *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + n);
-        const float4 wu =
-            *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + inter + n);
-        const int g[4] = {acc[t][s][0], acc[t][s][1], acc[t][s][2], acc[t][s][3]};
-        const int u[4] = {acc[t + 1][s][0], acc[t + 1][s][1], acc[t + 1][s][2], acc[t + 1][s][3]};
-        *reinterpret_cast<uint2*>(out + (int64_t)tok[s] * inter + n) = silu_mul_epilogue4(g, u, as, wg, wu);
-      }
+      const int n = wrow[0] + 4 * grp;  // gate channel; up channel is n + inter
+      const float4 wg = *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + n);
+      const float4 wu = *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + inter + n);
+      const int g[4] = {acc[0][s][0], acc[0][s][1], acc[0][s][2], acc[0][s][3]};
+      const int u[4] = {acc[1][s][0], acc[1][s][1], acc[1][s][2], acc[1][s][3]};
+      *reinterpret_cast<uint2*>(out + (int64_t)tok[s] * inter + n) = silu_mul_epilogue4(g, u, as, wg, wu);
     }
   }
 }
 
 // grid.x: groups of kWaves wave-tiles along the weight rows; grid.y: 64-row (B-row) blocks.
-template <int MODE, int TPW>
-__global__ __launch_bounds__(kThreads) void gemm_stream_kernel(StreamParams p) {
+template <int MODE>
+__global__ __launch_bounds__(kThreads, 3) void gemm_stream_kernel(StreamParams p) {
+  constexpr int TPW = kTiles;
+  __shared__ __align__(16) char lds[kWaves * kWaveLds];
   const int blk = blockIdx.y;
   const int npp = *p.npp;
   if ((int64_t)blk * p.B >= npp) return;
@@ -215,16 +224,13 @@ __global__ __launch_bounds__(kThreads) void gemm_stream_kernel(StreamParams p) {
   const int nsub = (nvalid + kSub - 1) / kSub;
   for (int sub0 = 0; sub0 < nsub; sub0 += kGroup) {
     const int ns = nsub - sub0 < kGroup ? nsub - sub0 : kGroup;
-    switch (ns) {
-      case 1: stream_pass<MODE, TPW, 1>(p, blk, e, sub0, wrow, wok); break;
-      case 2: stream_pass<MODE, TPW, 2>(p, blk, e, sub0, wrow, wok); break;
-      case 3: stream_pass<MODE, TPW, 3>(p, blk, e, sub0, wrow, wok); break;
-      default: stream_pass<MODE, TPW, 4>(p, blk, e, sub0, wrow, wok); break;
-    }
+    char* wave_lds = lds + (threadIdx.x / kWave) * kWaveLds;
+    stream_pass<MODE, kGroup>(p, blk, e, sub0, wrow, wok, wave_lds);
+    (void)ns;
   }
 }
 
-template <int MODE, int TPW>
+template <int MODE>
 hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   StreamParams p;
   p.a_q = a.a_q;
@@ -243,13 +249,13 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   p.B = a.block_size;
   p.out = a.out;
   const int row_tiles = MODE == kGateUpSilu ? a.n / 2 / 16 : a.n / 16;
-  const int tiles_per_wave = MODE == kGateUpSilu ? TPW / 2 : TPW;
+  const int tiles_per_wave = MODE == kGateUpSilu ? kTiles / 2 : kTiles;
   const int wave_tiles = (row_tiles + tiles_per_wave - 1) / tiles_per_wave;
   const int64_t blocks = (a.sorted_cap + a.block_size - 1) / a.block_size;
   if (blocks == 0 || wave_tiles == 0) return hipSuccess;
   if (blocks > 65535) return hipErrorInvalidValue;
   const dim3 grid((unsigned)((wave_tiles + kWaves - 1) / kWaves), (unsigned)blocks);
-  hipLaunchKernelGGL((gemm_stream_kernel<MODE, TPW>), grid, dim3(kThreads), 0, stream, p);
+  hipLaunchKernelGGL(gemm_stream_kernel<MODE>, grid, dim3(kThreads), 0, stream, p);
   return hipGetLastError();
 }
 
@@ -257,9 +263,9 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
 
 hipError_t launch_gemm_stream(const GemmArgs& a, hipStream_t stream) {
   switch (a.mode) {
-    case kGateUpSilu: return launch_mode<kGateUpSilu, MOE_I8_STREAM_TPW>(a, stream);
-    case kDown: return launch_mode<kDown, MOE_I8_STREAM_TPW>(a, stream);
-    case kAccI32: return launch_mode<kAccI32, MOE_I8_STREAM_TPW>(a, stream);
+    case kGateUpSilu: return launch_mode<kGateUpSilu>(a, stream);
+    case kDown: return launch_mode<kDown>(a, stream);
+    case kAccI32: return launch_mode<kAccI32>(a, stream);
     default: return hipErrorInvalidValue;
   }
 }
