@@ -9,6 +9,7 @@
 // Small inputs run in one 1024-thread workgroup (histogram, scans and scatter fused).  Large
 // inputs use three launches: per-wave histograms, one scan workgroup, scatter.
 #include "common.hpp"
+#include "quant_body.hpp"
 
 namespace moe_i8 {
 namespace {
@@ -134,11 +135,10 @@ __device__ __forceinline__ void write_expert_ids(const int* seg, int E, int B, i
 }
 
 // LDS layout: hist[kSingleWaves][E] | seg[E + 1] | wave_sums[kSingleWaves + 1]
-__global__ __launch_bounds__(kSingleThreads) void align_single_kernel(
+__device__ __forceinline__ void align_single_body(
     const int32_t* __restrict__ ids, int P, int E, int B, int nbits,
     int32_t* __restrict__ sorted, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
-    int64_t expert_cap, int32_t* __restrict__ npp_out) {
-  extern __shared__ int smem[];
+    int64_t expert_cap, int32_t* __restrict__ npp_out, int* smem) {
   int* hist = smem;
   int* seg = hist + kSingleWaves * E;
   int* wave_sums = seg + E + 1;
@@ -180,6 +180,30 @@ __global__ __launch_bounds__(kSingleThreads) void align_single_kernel(
   write_expert_ids(seg, E, B, npp, expert_ids, expert_cap);
   __syncthreads();
   wave_scatter(mine, begin, end - begin, E, nbits, hist + wave * E, sorted, sorted_cap);
+}
+
+__global__ __launch_bounds__(kSingleThreads) void align_single_kernel(
+    const int32_t* __restrict__ ids, int P, int E, int B, int nbits,
+    int32_t* __restrict__ sorted, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
+    int64_t expert_cap, int32_t* __restrict__ npp_out) {
+  extern __shared__ int smem[];
+  align_single_body(ids, P, E, B, nbits, sorted, sorted_cap, expert_ids, expert_cap, npp_out, smem);
+}
+
+// One launch for small batches: workgroup 0 runs moe_align, every other workgroup quantises 16
+// activation rows (one per wavefront).  The two halves are independent.
+template <int VPL>
+__global__ __launch_bounds__(kSingleThreads) void align_quant_kernel(
+    const int32_t* __restrict__ ids, int P, int E, int B, int nbits,
+    int32_t* __restrict__ sorted, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
+    int64_t expert_cap, int32_t* __restrict__ npp_out, QuantArgs q) {
+  extern __shared__ int smem[];
+  if (blockIdx.x == 0) {
+    align_single_body(ids, P, E, B, nbits, sorted, sorted_cap, expert_ids, expert_cap, npp_out, smem);
+    return;
+  }
+  const int64_t row = (int64_t)(blockIdx.x - 1) * kSingleWaves + threadIdx.x / kWave;
+  if (row < q.rows) quant_one_row<VPL>(q, row);
 }
 
 // ---- multi-launch path -------------------------------------------------------------------
@@ -286,6 +310,41 @@ int64_t align_workspace_ints(int64_t num_pairs, int num_experts) {
   if (num_pairs <= kSingleMaxPairs) return 0;
   const int64_t units = (num_pairs + kMultiChunk - 1) / kMultiChunk;
   return 2 * units * num_experts + num_experts + 1;
+}
+
+bool align_quant_fusable(const AlignArgs& a, const QuantArgs& q) {
+  return a.num_pairs <= kSingleMaxPairs && q.rows > 0 && q.rows <= kSingleMaxPairs;
+}
+
+namespace {
+size_t single_lds_bytes(int E) { return sizeof(int) * ((size_t)kSingleWaves * E + E + 1 + kSingleWaves + 1); }
+constexpr int kSingleLdsMax = (int)(sizeof(int) * ((size_t)kSingleWaves * kMaxExperts + kMaxExperts + kSingleWaves + 2));
+}  // namespace
+
+hipError_t launch_align_quant(const AlignArgs& a, const QuantArgs& q, hipStream_t stream) {
+  const int E = a.num_experts;
+  const dim3 grid(1 + (unsigned)((q.rows + kSingleWaves - 1) / kSingleWaves));
+#define MOE_I8_FUSED_LAUNCH(V)                                                                      \
+  do {                                                                                              \
+    static const hipError_t attr = hipFuncSetAttribute((const void*)align_quant_kernel<V>,          \
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize,  \
+                                                       kSingleLdsMax);                              \
+    if (attr != hipSuccess) return attr;                                                            \
+    hipLaunchKernelGGL(align_quant_kernel<V>, grid, dim3(kSingleThreads), single_lds_bytes(E),      \
+                       stream, a.topk_ids, (int)a.num_pairs, E, a.block_size, bits_for(E),          \
+                       a.sorted_token_ids, a.sorted_cap, a.expert_ids, a.expert_cap,                \
+                       a.num_tokens_post_padded, q);                                                \
+  } while (0)
+  switch (quant_vectors_per_lane(q.cols)) {
+    case 1: MOE_I8_FUSED_LAUNCH(1); break;
+    case 2: MOE_I8_FUSED_LAUNCH(2); break;
+    case 4: MOE_I8_FUSED_LAUNCH(4); break;
+    case 8: MOE_I8_FUSED_LAUNCH(8); break;
+    case 16: MOE_I8_FUSED_LAUNCH(16); break;
+    default: MOE_I8_FUSED_LAUNCH(0); break;
+  }
+#undef MOE_I8_FUSED_LAUNCH
+  return hipGetLastError();
 }
 
 hipError_t launch_align(const AlignArgs& a, hipStream_t stream) {

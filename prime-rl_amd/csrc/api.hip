@@ -331,12 +331,41 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
   void* down = ws + c.down;
   const int64_t p = m * top_k;
 
-  if (int rc = moe_i8_quant_rows(hidden, MOE_I8_DTYPE_BF16, m, hidden_size, hidden_size, nullptr, 1, m,
-                                 x_q, a1, stream))
-    return rc;
-  if (int rc = moe_i8_align_block_size(topk_ids, p, num_experts, block_size, sorted, c.cap, eids, c.ecap,
-                                       npp, ws + c.align_ws, c.align_bytes, stream))
-    return rc;
+  // Small batches: moe_align (one workgroup) and the quantisation of the input share one launch.
+  moe_i8::AlignArgs aa;
+  aa.topk_ids = topk_ids;
+  aa.num_pairs = p;
+  aa.num_experts = num_experts;
+  aa.block_size = block_size;
+  aa.sorted_token_ids = sorted;
+  aa.sorted_cap = c.cap;
+  aa.expert_ids = eids;
+  aa.expert_cap = c.ecap;
+  aa.num_tokens_post_padded = npp;
+  aa.workspace = reinterpret_cast<int32_t*>(ws + c.align_ws);
+  moe_i8::QuantArgs qa;
+  qa.x = static_cast<const uint16_t*>(hidden);
+  qa.src_rows = m;
+  qa.cols = hidden_size;
+  qa.row_stride = hidden_size;
+  qa.gather = nullptr;
+  qa.gather_div = 1;
+  qa.rows = m;
+  qa.q = x_q;
+  qa.scale = a1;
+  if (num_experts >= 1 && num_experts <= MOE_I8_MAX_EXPERTS && aligned16(hidden) &&
+      moe_i8::align_quant_fusable(aa, qa)) {
+    if (int rc = check_launch(moe_i8::launch_align_quant(aa, qa, static_cast<hipStream_t>(stream)),
+                              "align_quant"))
+      return rc;
+  } else {
+    if (int rc = moe_i8_quant_rows(hidden, MOE_I8_DTYPE_BF16, m, hidden_size, hidden_size, nullptr, 1, m,
+                                   x_q, a1, stream))
+      return rc;
+    if (int rc = moe_i8_align_block_size(topk_ids, p, num_experts, block_size, sorted, c.cap, eids, c.ecap,
+                                         npp, ws + c.align_ws, c.align_bytes, stream))
+      return rc;
+  }
   if (int rc = moe_i8_gemm_gate_up_silu(x_q, a1, w1, w1_scale, sorted, eids, npp, p, top_k, num_experts,
                                         hidden_size, inter, block_size, c.cap, act, variant, stream))
     return rc;

@@ -97,6 +97,9 @@ struct QuantArgs {
   float* scale;
 };
 hipError_t launch_quant_rows(const QuantArgs& a, hipStream_t stream);
+// moe_align and the quantisation of `q` in one launch; only when align_quant_fusable() says so.
+bool align_quant_fusable(const AlignArgs& a, const QuantArgs& q);
+hipError_t launch_align_quant(const AlignArgs& a, const QuantArgs& q, hipStream_t stream);
 
 enum GemmMode { kGateUpSilu = 0, kDown = 1, kAccI32 = 2 };
 

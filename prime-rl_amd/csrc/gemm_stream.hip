@@ -21,6 +21,9 @@
 // finds them in L2); sub-tiles that hold only padding are skipped (valid rows are a prefix of the
 // block).  Blocks with many rows belong to the LDS-tiled family.
 #include "common.hpp"
+#ifdef EXP_PPW_ENV
+#include <stdlib.h>
+#endif
 
 namespace moe_i8 {
 namespace {
@@ -51,6 +54,7 @@ struct StreamParams {
   int N;
   int K;
   int B;
+  int pairs_per_wave;  // consecutive tile pairs one wavefront streams back to back
   void* out;
 };
 
@@ -60,10 +64,29 @@ struct Window {
   v4i a[NS][kWinSteps];
 };
 
+// Rows of the q-th tile pair of the weight matrix: (gate tile, matching up tile) for gate_up,
+// two consecutive tiles otherwise.  An invalid tile points at row 0 and is never stored.
+template <int MODE>
+__device__ __forceinline__ void pair_rows(const StreamParams& p, int q, int (&wrow)[kTiles], bool (&wok)[kTiles]) {
+  if constexpr (MODE == kGateUpSilu) {
+    const int inter = p.N / 2;
+    const int ch = q * 16;
+    wok[0] = wok[1] = ch < inter;
+    wrow[0] = wok[0] ? ch : 0;
+    wrow[1] = wok[0] ? inter + ch : 0;
+  } else {
+#pragma unroll
+    for (int t = 0; t < kTiles; ++t) {
+      const int ch = (q * kTiles + t) * 16;
+      wok[t] = ch < p.N;
+      wrow[t] = wok[t] ? ch : 0;
+    }
+  }
+}
+
 template <int MODE, int NS>
-__device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int e, int sub0,
-                                            const int (&wrow)[kTiles], const bool (&wok)[kTiles],
-                                            char* wave_lds) {
+__device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int e, int sub0, int first_pair,
+                                            int npairs, char* wave_lds) {
   const int lane = lane_id();
   const int col = lane & 15;  // token slot inside a sub-tile / weight row inside a tile
   const int grp = lane >> 4;  // which 16 reduction bytes of each step; which 4 output channels
@@ -82,10 +105,7 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
   // Load j of a window covers rows 4 * (j % 4) + (lane >> 4) of tile j / 4, chunk lane & 15.
   const int ld_row = lane >> 4;
   const int ld_chunk = lane & 15;
-  const int8_t* wp[kTiles];
-#pragma unroll
-  for (int t = 0; t < kTiles; ++t)
-    wp[t] = p.w + ((int64_t)e * p.N + wrow[t] + ld_row) * K + ld_chunk * 16;
+  const int8_t* wbase = p.w + ((int64_t)e * p.N + ld_row) * K + ld_chunk * 16;
   // LDS: [32 rows][256 B]; chunk c of row r sits at position c ^ (r & 15)
   const int st_base = ld_row * kWinBytes + ((ld_chunk ^ ld_row) * 16);  // ^ (j % 4) * 64, + j * 1024
   const int rd_base = col * kWinBytes + ((grp ^ col) * 16);             // ^ u * 64, + t * 4096
@@ -96,20 +116,83 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
 #pragma unroll
     for (int s = 0; s < NS; ++s) acc[t][s] = v4i{0, 0, 0, 0};
 
-  auto fetch = [&](Window<NS>& win, int k0) {
-    const bool chunk_in = k0 + ld_chunk * 16 < K;  // only the last window of a ragged K is partial
+  // The wavefront walks windows (pair 0, k 0), (pair 0, k 256), ..., (pair 1, k 0), ... ; `fq`/`fk`
+  // track the window being fetched, `cq`/`ck` the one being consumed.
+  int fq = 0, fk = 0;
+  auto fetch = [&](Window<NS>& win) {
+    int wrow[kTiles];
+    bool wok[kTiles];
+    pair_rows<MODE>(p, first_pair + fq, wrow, wok);
+    const bool chunk_in = fk + ld_chunk * 16 < K;  // only the last window of a ragged K is partial
 #pragma unroll
     for (int j = 0; j < kWinLoads; ++j) {
-      const int8_t* src = wp[j / 4] + (int64_t)(4 * (j % 4)) * K + k0;
+      const int8_t* src = wbase + (int64_t)(wrow[j / 4] + 4 * (j % 4)) * K + fk;
       win.w[j] = chunk_in ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src)) : v4i{0, 0, 0, 0};
     }
 #pragma unroll
     for (int s = 0; s < NS; ++s)
 #pragma unroll
       for (int u = 0; u < kWinSteps; ++u)
-        win.a[s][u] = k0 + u * kStepK < K ? *reinterpret_cast<const v4i*>(ap[s] + k0 + u * kStepK)
+        win.a[s][u] = fk + u * kStepK < K ? *reinterpret_cast<const v4i*>(ap[s] + fk + u * kStepK)
                                            : v4i{0, 0, 0, 0};
+    fk += kWinBytes;
+    if (fk >= K) {
+      fk = 0;
+      ++fq;
+    }
   };
+
+  // Epilogue of one tile pair: lane holds channels wrow[t] + 4 * grp + {0..3} of token tok[s].
+  auto finish_pair = [&](int q) {
+    int wrow[kTiles];
+    bool wok[kTiles];
+    pair_rows<MODE>(p, first_pair + q, wrow, wok);
+    if constexpr (MODE == kAccI32) {
+      int32_t* out = static_cast<int32_t*>(p.out);
+#pragma unroll
+      for (int t = 0; t < kTiles; ++t)
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+          if (wok[t] && tok_ok[s])
+            *reinterpret_cast<v4i*>(out + (int64_t)tok[s] * p.N + wrow[t] + 4 * grp) = acc[t][s];
+    } else if constexpr (MODE == kDown) {
+      uint16_t* out = static_cast<uint16_t*>(p.out);
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        if (!tok_ok[s]) continue;
+        const float as = p.a_scale[tok[s] / p.row_div];
+        const float rw = p.row_weight[tok[s]];
+#pragma unroll
+        for (int t = 0; t < kTiles; ++t) {
+          if (!wok[t]) continue;
+          const int n = wrow[t] + 4 * grp;
+          const float4 ws = *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + n);
+          const int v[4] = {acc[t][s][0], acc[t][s][1], acc[t][s][2], acc[t][s][3]};
+          *reinterpret_cast<uint2*>(out + (int64_t)tok[s] * p.N + n) = down_epilogue4(v, as, ws, rw);
+        }
+      }
+    } else {  // kGateUpSilu: tile 0 is gate, tile 1 the matching up rows; out is [P, N / 2]
+      uint16_t* out = static_cast<uint16_t*>(p.out);
+      const int inter = p.N / 2;
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        if (!tok_ok[s] || !wok[0]) continue;
+        const float as = p.a_scale[tok[s] / p.row_div];
+        const int n = wrow[0] + 4 * grp;  // gate channel; up channel is n + inter
+        const float4 wg = *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + n);
+        const float4 wu = *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + inter + n);
+        const int g[4] = {acc[0][s][0], acc[0][s][1], acc[0][s][2], acc[0][s][3]};
+        const int u[4] = {acc[1][s][0], acc[1][s][1], acc[1][s][2], acc[1][s][3]};
+        *reinterpret_cast<uint2*>(out + (int64_t)tok[s] * inter + n) = silu_mul_epilogue4(g, u, as, wg, wu);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < kTiles; ++t)
+#pragma unroll
+      for (int s = 0; s < NS; ++s) acc[t][s] = v4i{0, 0, 0, 0};
+  };
+
+  int cq = 0, ck = 0;
   auto consume = [&](const Window<NS>& win) {
 #pragma unroll
     for (int j = 0; j < kWinLoads; ++j)
@@ -126,64 +209,30 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
         for (int s = 0; s < NS; ++s)
           acc[t][s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(frag[t], win.a[s][u], acc[t][s], 0, 0, 0);
     }
+    ck += kWinBytes;
+    if (ck >= K) {
+      finish_pair(cq);
+      ck = 0;
+      ++cq;
+    }
   };
 
+  const int nwin = (K + kWinBytes - 1) / kWinBytes;
+  const int total = npairs * nwin;
   Window<NS> w0, w1;
-  fetch(w0, 0);
-  for (int k0 = 0; k0 < K; k0 += 2 * kWinBytes) {
-    if (k0 + kWinBytes < K) fetch(w1, k0 + kWinBytes);
+  fetch(w0);
+  for (int i = 0; i < total; i += 2) {
+    if (i + 1 < total) fetch(w1);
     consume(w0);
-    if (k0 + kWinBytes >= K) break;
-    if (k0 + 2 * kWinBytes < K) fetch(w0, k0 + 2 * kWinBytes);
+    if (i + 1 >= total) break;
+    if (i + 2 < total) fetch(w0);
     consume(w1);
-  }
-
-  // Epilogue: lane holds channels wrow[t] + 4 * grp + {0..3} of token tok[s].
-  if constexpr (MODE == kAccI32) {
-    int32_t* out = static_cast<int32_t*>(p.out);
-#pragma unroll
-    for (int t = 0; t < kTiles; ++t)
-#pragma unroll
-      for (int s = 0; s < NS; ++s)
-        if (wok[t] && tok_ok[s])
-          *reinterpret_cast<v4i*>(out + (int64_t)tok[s] * p.N + wrow[t] + 4 * grp) = acc[t][s];
-  } else if constexpr (MODE == kDown) {
-    uint16_t* out = static_cast<uint16_t*>(p.out);
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      if (!tok_ok[s]) continue;
-      const float as = p.a_scale[tok[s] / p.row_div];
-      const float rw = p.row_weight[tok[s]];
-#pragma unroll
-      for (int t = 0; t < kTiles; ++t) {
-        if (!wok[t]) continue;
-        const int n = wrow[t] + 4 * grp;
-        const float4 ws = *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + n);
-        const int v[4] = {acc[t][s][0], acc[t][s][1], acc[t][s][2], acc[t][s][3]};
-        *reinterpret_cast<uint2*>(out + (int64_t)tok[s] * p.N + n) = down_epilogue4(v, as, ws, rw);
-      }
-    }
-  } else {  // kGateUpSilu: tile 0 is gate, tile 1 the matching up rows; out is [P, N / 2]
-    uint16_t* out = static_cast<uint16_t*>(p.out);
-    const int inter = p.N / 2;
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      if (!tok_ok[s] || !wok[0]) continue;
-      const float as = p.a_scale[tok[s] / p.row_div];
-      const int n = wrow[0] + 4 * grp;  // gate channel; up channel is n + inter
-      const float4 wg = *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + n);
-      const float4 wu = *reinterpret_cast<const float4*>(p.w_scale + (int64_t)e * p.N + inter + n);
-      const int g[4] = {acc[0][s][0], acc[0][s][1], acc[0][s][2], acc[0][s][3]};
-      const int u[4] = {acc[1][s][0], acc[1][s][1], acc[1][s][2], acc[1][s][3]};
-      *reinterpret_cast<uint2*>(out + (int64_t)tok[s] * inter + n) = silu_mul_epilogue4(g, u, as, wg, wu);
-    }
   }
 }
 
-// grid.x: groups of kWaves wave-tiles along the weight rows; grid.y: 64-row (B-row) blocks.
+// grid.x: groups of kWaves wavefronts along the weight rows; grid.y: 64-row (B-row) blocks.
 template <int MODE>
 __global__ __launch_bounds__(kThreads, 3) void gemm_stream_kernel(StreamParams p) {
-  constexpr int TPW = kTiles;
   __shared__ __align__(16) char lds[kWaves * kWaveLds];
   const int blk = blockIdx.y;
   const int npp = *p.npp;
@@ -191,28 +240,10 @@ __global__ __launch_bounds__(kThreads, 3) void gemm_stream_kernel(StreamParams p
   const int e = p.expert_ids[blk];
   if (e < 0 || e >= p.E) return;
   const int lane = lane_id();
-  const int wt = blockIdx.x * kWaves + threadIdx.x / kWave;
-
-  int wrow[TPW];
-  bool wok[TPW];
-  if constexpr (MODE == kGateUpSilu) {
-    const int inter = p.N / 2;
-#pragma unroll
-    for (int t = 0; t < TPW; t += 2) {
-      const int ch = (wt * (TPW / 2) + t / 2) * 16;
-      wok[t] = wok[t + 1] = ch < inter;
-      wrow[t] = wok[t] ? ch : 0;
-      wrow[t + 1] = wok[t] ? inter + ch : 0;
-    }
-  } else {
-#pragma unroll
-    for (int t = 0; t < TPW; ++t) {
-      const int ch = (wt * TPW + t) * 16;
-      wok[t] = ch < p.N;
-      wrow[t] = wok[t] ? ch : 0;
-    }
-  }
-  if (!wok[0]) return;
+  const int total_pairs = MODE == kGateUpSilu ? p.N / 2 / 16 : (p.N / 16 + kTiles - 1) / kTiles;
+  const int first_pair = (blockIdx.x * kWaves + threadIdx.x / kWave) * p.pairs_per_wave;
+  if (first_pair >= total_pairs) return;
+  const int npairs = total_pairs - first_pair < p.pairs_per_wave ? total_pairs - first_pair : p.pairs_per_wave;
 
   // Valid rows are a prefix of the block: count them to know how many sub-tiles to run.
   int nvalid = 0;
@@ -222,12 +253,9 @@ __global__ __launch_bounds__(kThreads, 3) void gemm_stream_kernel(StreamParams p
     nvalid += __popcll(__ballot(t >= 0 && t < p.P));
   }
   const int nsub = (nvalid + kSub - 1) / kSub;
-  for (int sub0 = 0; sub0 < nsub; sub0 += kGroup) {
-    const int ns = nsub - sub0 < kGroup ? nsub - sub0 : kGroup;
-    char* wave_lds = lds + (threadIdx.x / kWave) * kWaveLds;
-    stream_pass<MODE, kGroup>(p, blk, e, sub0, wrow, wok, wave_lds);
-    (void)ns;
-  }
+  char* wave_lds = lds + (threadIdx.x / kWave) * kWaveLds;
+  for (int sub0 = 0; sub0 < nsub; sub0 += kGroup)
+    stream_pass<MODE, kGroup>(p, blk, e, sub0, first_pair, npairs, wave_lds);
 }
 
 template <int MODE>
@@ -248,13 +276,19 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   p.K = a.k;
   p.B = a.block_size;
   p.out = a.out;
-  const int row_tiles = MODE == kGateUpSilu ? a.n / 2 / 16 : a.n / 16;
-  const int tiles_per_wave = MODE == kGateUpSilu ? kTiles / 2 : kTiles;
-  const int wave_tiles = (row_tiles + tiles_per_wave - 1) / tiles_per_wave;
+  const int total_pairs = MODE == kGateUpSilu ? a.n / 2 / 16 : (a.n / 16 + kTiles - 1) / kTiles;
+  // One tile pair per wavefront measured best in the decode regime (more wavefronts in flight beat
+  // longer streams per wavefront); the kernel itself handles any number of consecutive pairs.
+  int ppw = 1;
+#ifdef EXP_PPW_ENV
+  if (const char* env = getenv("EXP_PPW")) ppw = atoi(env);
+#endif
+  p.pairs_per_wave = ppw;
+  const int waves = (total_pairs + ppw - 1) / ppw;
   const int64_t blocks = (a.sorted_cap + a.block_size - 1) / a.block_size;
-  if (blocks == 0 || wave_tiles == 0) return hipSuccess;
+  if (blocks == 0 || waves == 0) return hipSuccess;
   if (blocks > 65535) return hipErrorInvalidValue;
-  const dim3 grid((unsigned)((wave_tiles + kWaves - 1) / kWaves), (unsigned)blocks);
+  const dim3 grid((unsigned)((waves + kWaves - 1) / kWaves), (unsigned)blocks);
   hipLaunchKernelGGL(gemm_stream_kernel<MODE>, grid, dim3(kThreads), 0, stream, p);
   return hipGetLastError();
 }
