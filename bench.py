@@ -34,15 +34,17 @@ SWEEP_M = (16, 128, 1024, 8192)
 
 
 def _profile_traffic(kernel: str, M: int):
-    """HBM bytes per launch measured with rocprofv3 --pmc, when a summary for this kernel and batch
-    size has been recorded in profiles/traffic.json; otherwise None."""
-    path = ROOT / "profiles" / "traffic.json"
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE, each scaled by
+    what the counter reads for a plain copy of known size), when a summary for this kernel and batch
+    size has been recorded under profiles/; otherwise None."""
+    path = ROOT / "profiles" / "hbm_traffic_gate_up.txt"
     if not path.exists():
         return None
-    try:
-        return json.loads(path.read_text()).get(f"{kernel}@M={M}")
-    except (ValueError, OSError):
-        return None
+    for line in path.read_text().splitlines():
+        f = line.split()
+        if len(f) == 7 and f[0] == "traffic" and f[1] == kernel and f[2] == f"M={M}":
+            return (float(f[3]) * float(f[5]) + float(f[4]) * float(f[6])) * 1024.0
+    return None
 
 
 def build_workload(pkg, torch, shape_name: str, M: int, copies: int, seed: int):
