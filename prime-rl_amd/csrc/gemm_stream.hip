@@ -21,9 +21,6 @@
 // finds them in L2); sub-tiles that hold only padding are skipped (valid rows are a prefix of the
 // block).  Blocks with many rows belong to the LDS-tiled family.
 #include "common.hpp"
-#ifdef EXP_PPW_ENV
-#include <stdlib.h>
-#endif
 
 namespace moe_i8 {
 namespace {
@@ -279,10 +276,7 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   const int total_pairs = MODE == kGateUpSilu ? a.n / 2 / 16 : (a.n / 16 + kTiles - 1) / kTiles;
   // One tile pair per wavefront measured best in the decode regime (more wavefronts in flight beat
   // longer streams per wavefront); the kernel itself handles any number of consecutive pairs.
-  int ppw = 1;
-#ifdef EXP_PPW_ENV
-  if (const char* env = getenv("EXP_PPW")) ppw = atoi(env);
-#endif
+  const int ppw = 1;
   p.pairs_per_wave = ppw;
   const int waves = (total_pairs + ppw - 1) / ppw;
   const int64_t blocks = (a.sorted_cap + a.block_size - 1) / a.block_size;
