@@ -212,12 +212,14 @@ struct TileReads {
 
 __device__ __forceinline__ void multiply_stage(const TileReads& rd, const char* stage, v16i (&acc)[4][2]) {
   v4i a[4][4], b[4][2];
+  // reads in the order the MFMAs consume them: b0 a0 | b1 | a1 | a2 | a3 per 32-byte sub-step
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk) {
+    b[kk][0] = *reinterpret_cast<const v4i*>(stage + rd.x_ld[0] + rd.chunk[kk]);
+    a[kk][0] = *reinterpret_cast<const v4i*>(stage + rd.w_ld[0] + rd.chunk[kk]);
+    b[kk][1] = *reinterpret_cast<const v4i*>(stage + rd.x_ld[1] + rd.chunk[kk]);
 #pragma unroll
-    for (int tj = 0; tj < 2; ++tj) b[kk][tj] = *reinterpret_cast<const v4i*>(stage + rd.x_ld[tj] + rd.chunk[kk]);
-#pragma unroll
-    for (int ci = 0; ci < 4; ++ci) a[kk][ci] = *reinterpret_cast<const v4i*>(stage + rd.w_ld[ci] + rd.chunk[kk]);
+    for (int ci = 1; ci < 4; ++ci) a[kk][ci] = *reinterpret_cast<const v4i*>(stage + rd.w_ld[ci] + rd.chunk[kk]);
   }
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk)
@@ -226,13 +228,24 @@ __device__ __forceinline__ void multiply_stage(const TileReads& rd, const char* 
 #pragma unroll
       for (int tj = 0; tj < 2; ++tj)
         acc[ci][tj] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[kk][ci], b[kk][tj], acc[ci][tj], 0, 0, 0);
-  // operand reads of two sub-steps first, then MFMAs interleaved with the remaining reads
-  __builtin_amdgcn_sched_group_barrier(0x100, 12, 0);
-  __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
-  __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
-  __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
-  __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
-  __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
+  // Fine interleave, one group ahead: the first MFMA issues as soon as three operands are in and
+  // every later read is issued at least one MFMA group before its first use, so it is hidden
+  // behind MFMAs already queued (8 wavefronts share the LDS: a long burst of reads in front of the
+  // first MFMA would leave the matrix pipe idle at the start of every step).
+  __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);  // b0 a0 b1 of sub-step 0
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // a0 b0
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // a1
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // a0 b1
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // a2
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // a1
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // a3
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // a2
+    if (kk < 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // next b0 a0
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // a3
+    if (kk < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // next b1
+  }
 }
 
 // acc[ci][tj][4q + r] is channel base(ci) + 8q + 4 * (lane >> 5) + r of token row
