@@ -58,8 +58,9 @@ int run_gemm(const moe_i8::GemmArgs& g, int variant, hipStream_t stream) {
   } else if (variant == MOE_I8_GEMM_STREAM) {
     tile = false;
   } else {
-    // More than ~16 routed rows per expert on average: weights are reused enough for LDS tiles.
-    tile = moe_i8::gemm_tile_supports(g) && g.num_pairs > (int64_t)16 * g.num_experts;
+    // Measured crossover on the Qwen3-30B-A3B shape: the streaming family wins while a block holds
+    // one 16-row sub-tile (about 8 routed rows per expert), the LDS-tiled family from about 16 up.
+    tile = moe_i8::gemm_tile_supports(g) && g.num_pairs > (int64_t)12 * g.num_experts;
   }
   return check_launch(tile ? moe_i8::launch_gemm_tile(g, stream) : moe_i8::launch_gemm_stream(g, stream),
                       tile ? "gemm_tile" : "gemm_stream");
