@@ -109,6 +109,28 @@ def gate_up_work(shape, M: int, topk_ids):
     return ops, nbytes, n_act
 
 
+def time_weight_requant(pkg, torch, shape, steps: int, warmup: int) -> dict:
+    """Trainer bf16 expert weights of the whole layer → int8 kernel layout, written in place into the
+    engine's tensors (what happens to every MoE layer after each policy step).  HBM-bound: 2 bytes
+    read and 1 written per weight, plus one fp32 scale per output channel."""
+    E, I, H = shape.E_total, shape.I, shape.H
+    g = torch.Generator(device="cuda:0").manual_seed(1)
+    gate, up = (torch.randn(E, I, H, generator=g, device="cuda:0").mul_(0.02).to(torch.bfloat16) for _ in range(2))
+    down = torch.randn(E, H, I, generator=g, device="cuda:0").mul_(0.02).to(torch.bfloat16)
+    params = pkg.quantize_expert_weights(gate, up, down)
+    for _ in range(warmup):
+        pkg.quantize_expert_weights(gate, up, down, out=params)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        pkg.quantize_expert_weights(gate, up, down, out=params)
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / steps
+    nbytes = 3 * E * I * H * 3 + 4 * E * (2 * I + H)
+    return {"us": t * 1e6, "bytes": nbytes, "hbm_gbps": nbytes / t / 1e9, "hbm_frac": nbytes / t / PEAK_HBM_BPS,
+            "layers_per_s": 1.0 / t}
+
+
 def cpu_baseline(oracle, torch, base, sample_m: int) -> dict:
     m = min(sample_m, base.hidden_states.shape[0])
     args = (base.hidden_states[:m], base.w1, base.w2, base.topk_weights[:m], base.topk_ids[:m],
@@ -221,6 +243,9 @@ def main() -> int:
         "layer_hbm_frac": headline["layer_hbm_frac"],
         "sweep": sweep,
     }
+    if not args.no_sweep:
+        out["weight_requant"] = time_weight_requant(pkg, torch, pkg.inputs.SHAPES[args.shape],
+                                                    max(args.steps // 2, 1), max(args.warmup // 2, 1))
     if not args.no_cpu:
         oracle = importlib.import_module("oracle.moe_i8_oracle")
         out["cpu_baseline"] = cpu_baseline(oracle, torch, base_headline, args.cpu_sample)

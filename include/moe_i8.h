@@ -78,6 +78,22 @@ int moe_i8_quant_rows(const void* x, int dtype, int64_t src_rows, int64_t cols, 
                       void* stream);
 
 /*
+ * Per-output-channel symmetric int8 quantisation of bf16 expert weights into the kernel layout,
+ * for in-place updates of a quantised engine after a policy step: the int8 analogue of the
+ * reference's `quantize_to_vllm_kernel_format` (src/prime_rl/trainer/models/fp8.py:5-64: scale =
+ * absmax / qmax clamped from below, q = w / scale) + `torch.cat([gate, up], dim=1)`
+ * (src/prime_rl/trainer/models/glm_moe_dsa/converting_glm_moe_dsa.py:97-104) feeding the in-place
+ * `param.copy_` of src/prime_rl/inference/vllm/worker/weight_transfer.py:97-134.
+ * w bf16 [rows, cols] -> q int8 and scale fp32 at output row
+ * (r / rows_per_group) * out_rows_per_group + out_row_offset + r % rows_per_group
+ * (rows_per_group == 0: output row == r); scale = max(absmax / 127, 1e-12),
+ * q = clamp(rint(w / scale), -127, 127) with ties to even.
+ */
+int moe_i8_quant_weights(const void* w, int dtype, int64_t rows, int64_t cols, int64_t rows_per_group,
+                         int64_t out_rows_per_group, int64_t out_row_offset, int8_t* q, float* scale,
+                         void* stream);
+
+/*
  * Replaces vLLM `fused_moe_kernel` (gate_up GEMM, use_int8_w8a8, per-channel) +
  * `silu_and_mul` (csrc/activation_kernels.cu).  In-tree semantics: grouped GEMM
  * contract tests/unit/train/models/test_moe.py:60-66; gate-then-up stacking

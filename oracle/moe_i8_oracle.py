@@ -25,6 +25,13 @@ Pinning status (what independent evidence each function is checked against in
   reference's own activation (``trainer/models/layers/activations.py:29-34``).
 * ``moe_sum`` / combine      pinned: the reference's dispatcher known answer
   (``tests/unit/train/models/test_moe.py:83-109``) and closed form.
+* ``quantize_weights_per_channel`` / ``quantize_expert_weights``  layout pinned by the
+  shapes the reference's conversion test asserts
+  (``tests/unit/train/models/test_glm_moe_dsa_conversion.py:47-50,65-68``) and by ``torch.cat``;
+  arithmetic pinned by a tie vector, zero rows, the half-step error bound and an element-wise
+  brute force in numpy float32.  Parity unpinned against an int8 checkpoint producer: the
+  reference tree quantises weights to FP8 only (``trainer/models/fp8.py:5-41``); the int8
+  rule here is that function with qmax = 127, a whole row as the block and the integer grid.
 * ``fused_experts`` (whole)  parity unpinned at the vLLM boundary: no test or
   fixture in the reference touches int8 ``fused_experts``.  Pinned only against
   ``native_w8a8_moe`` (an independent per-expert formulation) and against the
@@ -52,6 +59,8 @@ __all__ = [
     "dequant_fp32_moe",
     "softmax_topk",
     "grouped_topk",
+    "quantize_weights_per_channel",
+    "quantize_expert_weights",
 ]
 
 
@@ -345,3 +354,34 @@ def grouped_topk(
         w = w / (w.sum(dim=-1, keepdim=True) + 1e-20)
     w = w * routed_scaling_factor
     return w.to(torch.float32), ids.to(torch.int32)
+
+
+# --------------------------------------------------------------------------- #
+# Weight (re)quantisation into the kernel layout
+# --------------------------------------------------------------------------- #
+def quantize_weights_per_channel(w: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Symmetric per-output-channel int8 quantisation of ``w [..., N, K]`` (one scale per row).
+
+    The reference's ``quantize_to_fp8_blockwise`` (``trainer/models/fp8.py:33-36``) with the block
+    widened to one whole row, ``qmax = 127`` and the integer grid: ``scale = (absmax / 127)
+    .clamp(min=1e-12)``; ``q = (w.float() / scale).clamp(-127, 127)`` rounded to nearest, ties to
+    even (what the cast to the quantised type does there).  Returns ``(q int8, scale fp32 [..., N])``.
+    """
+    wf = w.to(torch.float32)
+    absmax = wf.abs().amax(dim=-1, keepdim=True)
+    scale = (absmax / 127.0).clamp(min=1e-12)
+    q = torch.round(wf / scale).clamp(-127, 127).to(torch.int8)
+    return q, scale.squeeze(-1)
+
+
+def quantize_expert_weights(gate_proj: torch.Tensor, up_proj: torch.Tensor, down_proj: torch.Tensor):
+    """Trainer expert weights → the four tensors ``fused_experts`` consumes.
+
+    ``gate_proj, up_proj [E, I, H]``, ``down_proj [E, H, I]`` (the reference's ``w1, w3, w2``) →
+    ``w13 int8 [E, 2I, H]`` with gate rows first (``torch.cat([w1, w3], dim=1)``,
+    ``trainer/models/glm_moe_dsa/converting_glm_moe_dsa.py:97-104``), ``w13_scale fp32 [E, 2I]``,
+    ``w2 int8 [E, H, I]``, ``w2_scale fp32 [E, H]``.
+    """
+    w13, s13 = quantize_weights_per_channel(torch.cat([gate_proj, up_proj], dim=1))
+    w2, s2 = quantize_weights_per_channel(down_proj)
+    return w13, s13, w2, s2

@@ -14,6 +14,8 @@ from .api import (  # noqa: F401
     moe_align_block_size,
     moe_sum,
     per_token_quant_int8,
+    quantize_expert_weights,
+    quantize_weights_per_channel,
     sorted_capacity,
     workspace_bytes,
 )
@@ -23,6 +25,8 @@ __all__ = [
     "fused_experts",
     "moe_align_block_size",
     "per_token_quant_int8",
+    "quantize_weights_per_channel",
+    "quantize_expert_weights",
     "moe_sum",
     "gemm_gate_up_silu",
     "gemm_down",

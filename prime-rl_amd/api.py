@@ -20,6 +20,8 @@ __all__ = [
     "fused_experts",
     "moe_align_block_size",
     "per_token_quant_int8",
+    "quantize_weights_per_channel",
+    "quantize_expert_weights",
     "moe_sum",
     "gemm_gate_up_silu",
     "gemm_down",
@@ -146,6 +148,100 @@ def per_token_quant_int8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
         )
     )
     return q, scale
+
+
+def _quant_weights_into(w, q, scale, rows_per_group=0, out_rows_per_group=0, out_row_offset=0) -> None:
+    cols = w.shape[-1]
+    rows = w.numel() // cols if cols else 0
+    _abi.check(
+        _abi.load().moe_i8_quant_weights(
+            _ptr(w), _abi.DTYPE_BF16, rows, cols, rows_per_group, out_rows_per_group, out_row_offset,
+            _ptr(q), _ptr(scale), _stream(w),
+        )
+    )
+
+
+def _check_bf16_weight(name: str, w: torch.Tensor, ndim_min: int = 2) -> None:
+    _require_gpu(name, w)
+    if w.dtype != torch.bfloat16:
+        raise NotImplementedError(f"only bfloat16 weights are supported, got {w.dtype} for {name}")
+    if w.dim() < ndim_min:
+        raise ValueError(f"{name} must have at least {ndim_min} dimensions")
+    if w.shape[-1] == 0 or w.shape[-1] % 8:
+        raise ValueError(f"last dimension of {name} must be a positive multiple of 8")
+
+
+def quantize_weights_per_channel(
+    w: torch.Tensor, out: tuple[torch.Tensor, torch.Tensor] | None = None
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """Symmetric per-output-channel int8 quantisation of bf16 ``w [..., N, K]``: the reference's
+    blockwise weight quantiser (``src/prime_rl/trainer/models/fp8.py:33-36``) with one whole row as
+    the block and ``qmax = 127`` — ``scale = max(absmax / 127, 1e-12)``, ``q = rint(w / scale)``
+    clamped to ±127.  Returns ``(q int8 like w, scale fp32 [..., N])``; with ``out=(q, scale)`` the
+    result is written into those tensors (an in-place update of engine parameters, as
+    ``src/prime_rl/inference/vllm/worker/weight_transfer.py:97-134`` does with ``param.copy_``)."""
+    _check_bf16_weight("w", w)
+    if out is None:
+        q = torch.empty(w.shape, dtype=torch.int8, device=w.device)
+        scale = torch.empty(w.shape[:-1], dtype=torch.float32, device=w.device)
+    else:
+        q, scale = out
+        _require_gpu("out[0]", q)
+        _require_gpu("out[1]", scale)
+        if q.dtype != torch.int8 or q.shape != w.shape:
+            raise ValueError("out[0] must be int8 with the shape of w")
+        if scale.dtype != torch.float32 or scale.numel() != w.numel() // w.shape[-1]:
+            raise ValueError("out[1] must be fp32 with one element per row of w")
+    _quant_weights_into(w, q, scale)
+    return q, scale
+
+
+def quantize_expert_weights(
+    gate_proj: torch.Tensor,
+    up_proj: torch.Tensor,
+    down_proj: torch.Tensor,
+    out: tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor] | None = None,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Trainer expert weights → the int8 kernel layout ``fused_experts`` reads, in three launches and
+    with no concatenated bf16 intermediate.
+
+    ``gate_proj, up_proj`` bf16 ``[E, I, H]`` and ``down_proj`` bf16 ``[E, H, I]`` (``w1, w3, w2`` of
+    ``src/prime_rl/trainer/models/glm_moe_dsa/converting_glm_moe_dsa.py:97-125``) → ``w13 int8
+    [E, 2I, H]`` (gate rows first, as ``torch.cat([w1, w3], dim=1)`` there), ``w13_scale fp32
+    [E, 2I]``, ``w2 int8 [E, H, I]``, ``w2_scale fp32 [E, H]``.  ``out=(w13, w13_scale, w2,
+    w2_scale)`` overwrites the parameters of a running engine in place.
+    """
+    _check_bf16_weight("gate_proj", gate_proj, 3)
+    _check_bf16_weight("up_proj", up_proj, 3)
+    _check_bf16_weight("down_proj", down_proj, 3)
+    if gate_proj.dim() != 3 or gate_proj.shape != up_proj.shape:
+        raise ValueError("gate_proj and up_proj must both be [E, I, H]")
+    E, I, H = gate_proj.shape
+    if down_proj.shape != (E, H, I):
+        raise ValueError(f"down_proj must be [E, H, I] = {(E, H, I)}, got {tuple(down_proj.shape)}")
+    dev = gate_proj.device
+    if out is None:
+        w13 = torch.empty((E, 2 * I, H), dtype=torch.int8, device=dev)
+        s13 = torch.empty((E, 2 * I), dtype=torch.float32, device=dev)
+        w2 = torch.empty((E, H, I), dtype=torch.int8, device=dev)
+        s2 = torch.empty((E, H), dtype=torch.float32, device=dev)
+    else:
+        w13, s13, w2, s2 = out
+        for name, t, dtype, numel in (
+            ("w13", w13, torch.int8, E * 2 * I * H),
+            ("w13_scale", s13, torch.float32, E * 2 * I),
+            ("w2", w2, torch.int8, E * H * I),
+            ("w2_scale", s2, torch.float32, E * H),
+        ):
+            _require_gpu(name, t)
+            if t.dtype != dtype or t.numel() != numel:
+                raise ValueError(f"out tensor {name} must be {dtype} with {numel} elements")
+        if w13.shape != (E, 2 * I, H) or w2.shape != (E, H, I):
+            raise ValueError("out weights must be w13 [E, 2I, H] and w2 [E, H, I]")
+    _quant_weights_into(gate_proj, w13, s13, I, 2 * I, 0)
+    _quant_weights_into(up_proj, w13, s13, I, 2 * I, I)
+    _quant_weights_into(down_proj, w2, s2)
+    return w13, s13, w2, s2
 
 
 def moe_sum(input: torch.Tensor, output: torch.Tensor) -> None:

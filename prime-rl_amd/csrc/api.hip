@@ -150,6 +150,36 @@ int moe_i8_quant_rows(const void* x, int dtype, int64_t src_rows, int64_t cols, 
   return check_launch(moe_i8::launch_quant_rows(a, static_cast<hipStream_t>(stream)), "quant_rows");
 }
 
+int moe_i8_quant_weights(const void* w, int dtype, int64_t rows, int64_t cols, int64_t rows_per_group,
+                         int64_t out_rows_per_group, int64_t out_row_offset, int8_t* q, float* scale,
+                         void* stream) {
+  if (dtype != MOE_I8_DTYPE_BF16) return fail(MOE_I8_EUNSUPPORTED, "only bf16 weights are supported");
+  if (rows < 0) return fail(MOE_I8_EINVAL, "negative row count");
+  if (rows == 0) return MOE_I8_OK;
+  if (!w || !q || !scale) return fail(MOE_I8_EINVAL, "null pointer");
+  if (cols < 8 || cols % 8 || cols > INT32_MAX)
+    return fail(MOE_I8_EINVAL, "cols (%lld) must be a positive multiple of 8", (long long)cols);
+  if (!aligned16(w) || (reinterpret_cast<uintptr_t>(q) & 7u))
+    return fail(MOE_I8_EINVAL, "w must be 16-byte and q 8-byte aligned");
+  if (rows_per_group < 0 || (rows_per_group > 0 && (rows % rows_per_group || out_row_offset < 0 ||
+                                                     out_row_offset + rows_per_group > out_rows_per_group)))
+    return fail(MOE_I8_EINVAL, "row groups must tile the input and fit inside the output groups");
+  moe_i8::QuantArgs a;
+  a.x = static_cast<const uint16_t*>(w);
+  a.src_rows = rows;
+  a.cols = (int)cols;
+  a.row_stride = cols;
+  a.gather = nullptr;
+  a.gather_div = 1;
+  a.rows = rows;
+  a.q = q;
+  a.scale = scale;
+  a.rows_per_group = rows_per_group;
+  a.out_rows_per_group = out_rows_per_group;
+  a.out_row_offset = out_row_offset;
+  return check_launch(moe_i8::launch_quant_weights(a, static_cast<hipStream_t>(stream)), "quant_weights");
+}
+
 int moe_i8_gemm_gate_up_silu(const int8_t* x_q, const float* a_scale, const int8_t* w1,
                              const float* w1_scale, const int32_t* sorted_token_ids,
                              const int32_t* expert_ids, const int32_t* num_tokens_post_padded,

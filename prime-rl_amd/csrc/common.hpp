@@ -95,8 +95,16 @@ struct QuantArgs {
   int64_t rows;
   int8_t* q;
   float* scale;
+  // Output row of input row r is (r / rows_per_group) * out_rows_per_group + out_row_offset +
+  // r % rows_per_group; rows_per_group == 0 means out row == r.  Lets one call drop the gate or
+  // the up projection of every expert into its half of a stacked [E, 2I, H] tensor.
+  int64_t rows_per_group = 0;
+  int64_t out_rows_per_group = 0;
+  int64_t out_row_offset = 0;
 };
 hipError_t launch_quant_rows(const QuantArgs& a, hipStream_t stream);
+// Per-output-channel weight quantisation (round to nearest even of w / scale, scale = absmax / 127).
+hipError_t launch_quant_weights(const QuantArgs& a, hipStream_t stream);
 // moe_align and the quantisation of `q` in one launch; only when align_quant_fusable() says so.
 bool align_quant_fusable(const AlignArgs& a, const QuantArgs& q);
 hipError_t launch_align_quant(const AlignArgs& a, const QuantArgs& q, hipStream_t stream);

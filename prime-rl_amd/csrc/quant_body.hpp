@@ -38,15 +38,82 @@ __device__ __forceinline__ uint2 quant8(const uint4& v, float inv) {
   return make_uint2(out[0], out[1]);
 }
 
+// Largest |x| of 8 packed bf16 as a float.  Without the sign bit, bf16 patterns order like unsigned
+// integers, so the maximum is taken on packed 16-bit lanes (two elements per operation).
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float absmax8_packed(const uint4& v) {
+  const uint32_t w[4] = {v.x & 0x7fff7fffu, v.y & 0x7fff7fffu, v.z & 0x7fff7fffu, v.w & 0x7fff7fffu};
+  u16x2 m = __builtin_elementwise_max(
+      __builtin_elementwise_max(__builtin_bit_cast(u16x2, w[0]), __builtin_bit_cast(u16x2, w[1])),
+      __builtin_elementwise_max(__builtin_bit_cast(u16x2, w[2]), __builtin_bit_cast(u16x2, w[3])));
+  const uint32_t top = m[0] > m[1] ? m[0] : m[1];
+  return __uint_as_float(top << 16);
+}
+
+// Weight flavour of quant8: q = rint(x / scale) (ties to even, the correctly rounded fp32 quotient),
+// |q| <= 127 by construction of scale for finite weights.
+//
+// A correctly rounded division costs ~11 VALU operations per element.  Instead
+// fma(x, r, 1.5 * 2^23) rounds the exact product x * r to the nearest-even integer in ONE operation
+// (at that magnitude one ulp is 1) and leaves it as a two's complement byte in the low mantissa
+// bits.  It is evaluated for r = rcp(scale) * (1 -+ 2^-21): v_rcp_f32 is within 1 ulp, so the true
+// quotient and its fp32 rounding both lie between the two products, and rounding to an integer is
+// monotonic — when both give the same integer, that integer is the answer.  Only when they differ
+// (the quotient is within ~1e-4 of k + 0.5) is the vector redone with the true division.
+struct WeightRcp {
+  float scale, lo, hi;
+};
+__device__ __forceinline__ WeightRcp weight_rcp(float scale) {
+  const float r = __builtin_amdgcn_rcpf(scale);
+  return {scale, r * (1.0f - 0x1p-21f), r * (1.0f + 0x1p-21f)};
+}
+
+__device__ __forceinline__ uint2 quant8_weights(const uint4& v, const WeightRcp& s) {
+  constexpr float kMagic = 12582912.0f;  // 1.5 * 2^23
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  float x[8];
+  uint32_t y[8];
+  uint32_t differ = 0u;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    x[2 * i] = __uint_as_float(w[i] << 16);
+    x[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    y[i] = __float_as_uint(fmaf(x[i], s.lo, kMagic));
+    differ |= y[i] ^ __float_as_uint(fmaf(x[i], s.hi, kMagic));
+    asm("" : "+v"(differ));  // keeps this one xor-or per element (else it becomes 8 compares + a bit mask)
+  }
+  if (differ) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = __float_as_uint(rintf(x[i] / s.scale) + kMagic);
+  }
+  uint32_t out[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    // low bytes of four results -> one dword (selector: 0-3 = bytes of the 2nd operand, 4-7 = of the 1st)
+    const uint32_t p01 = __builtin_amdgcn_perm(y[4 * h + 1], y[4 * h], 0x0c0c0400u);
+    const uint32_t p23 = __builtin_amdgcn_perm(y[4 * h + 3], y[4 * h + 2], 0x04000c0cu);
+    out[h] = p01 | p23;
+  }
+  return make_uint2(out[0], out[1]);
+}
+
 // VPL = 16-byte vectors per lane held in registers (covers cols <= VPL * 512).
 // VPL == 0: rows of any length, read twice (second read served by the caches).
-template <int VPL>
+// kWeights: per-output-channel weight quantisation instead of the activation arithmetic:
+// scale = max(absmax / 127, 1e-12), q = clamp(rint(x / scale), +-127).
+template <int VPL, bool kWeights = false>
 __device__ __forceinline__ void quant_one_row(const QuantArgs& a, int64_t row) {
   const int lane = lane_id();
   const int64_t src = a.gather ? (int64_t)(a.gather[row] / a.gather_div) : row;
   const bool have = src >= 0 && src < a.src_rows;
   const uint4* in = reinterpret_cast<const uint4*>(a.x + (have ? src : 0) * a.row_stride);
-  uint2* out = reinterpret_cast<uint2*>(a.q + row * (int64_t)a.cols);
+  const int64_t orow = a.rows_per_group > 0
+                           ? (row / a.rows_per_group) * a.out_rows_per_group + a.out_row_offset + row % a.rows_per_group
+                           : row;
+  uint2* out = reinterpret_cast<uint2*>(a.q + orow * (int64_t)a.cols);
   const int nvec = a.cols / kQuantVec;
 
   if constexpr (VPL > 0) {
@@ -59,23 +126,39 @@ __device__ __forceinline__ void quant_one_row(const QuantArgs& a, int64_t row) {
     float m = 0.0f;
 #pragma unroll
     for (int i = 0; i < VPL; ++i) m = fmaxf(m, absmax8(v[i]));
-    const float absmax = fmaxf(wave_max(m), 1e-10f);
-    const float inv = 127.0f / absmax;
-    if (lane == 0) a.scale[row] = absmax / 127.0f;
+    if constexpr (kWeights) {
+      const WeightRcp s = weight_rcp(fmaxf(wave_max(m) / 127.0f, 1e-12f));
+      if (lane == 0) a.scale[orow] = s.scale;
 #pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-      const int c = lane + i * kWave;
-      if (c < nvec) out[c] = quant8(v[i], inv);
+      for (int i = 0; i < VPL; ++i) {
+        const int c = lane + i * kWave;
+        if (c < nvec) out[c] = quant8_weights(v[i], s);
+      }
+    } else {
+      const float absmax = fmaxf(wave_max(m), 1e-10f);
+      const float inv = 127.0f / absmax;
+      if (lane == 0) a.scale[orow] = absmax / 127.0f;
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        const int c = lane + i * kWave;
+        if (c < nvec) out[c] = quant8(v[i], inv);
+      }
     }
   } else {
     float m = 0.0f;
     if (have)
       for (int c = lane; c < nvec; c += kWave) m = fmaxf(m, absmax8(in[c]));
-    const float absmax = fmaxf(wave_max(m), 1e-10f);
-    const float inv = 127.0f / absmax;
-    if (lane == 0) a.scale[row] = absmax / 127.0f;
-    for (int c = lane; c < nvec; c += kWave)
-      out[c] = have ? quant8(in[c], inv) : make_uint2(0u, 0u);
+    if constexpr (kWeights) {
+      const WeightRcp s = weight_rcp(fmaxf(wave_max(m) / 127.0f, 1e-12f));
+      if (lane == 0) a.scale[orow] = s.scale;
+      for (int c = lane; c < nvec; c += kWave) out[c] = have ? quant8_weights(in[c], s) : make_uint2(0u, 0u);
+    } else {
+      const float absmax = fmaxf(wave_max(m), 1e-10f);
+      const float inv = 127.0f / absmax;
+      if (lane == 0) a.scale[orow] = absmax / 127.0f;
+      for (int c = lane; c < nvec; c += kWave)
+        out[c] = have ? quant8(in[c], inv) : make_uint2(0u, 0u);
+    }
   }
 }
 

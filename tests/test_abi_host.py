@@ -63,6 +63,14 @@ def test_c_abi_rejects_bad_arguments_without_launching(pra):
     assert lib.moe_i8_quant_rows(p, 0, 4, 64, 32, None, 1, 4, p, p, None) == abi.EINVAL
     assert lib.moe_i8_quant_rows(None, 0, 4, 64, 64, None, 1, 4, p, p, None) == abi.EINVAL
     assert lib.moe_i8_quant_rows(p, 0, 4, 64, 64, None, 1, 0, p, p, None) == abi.OK  # zero rows: no-op
+    # weight quant: dtype, cols, row groups that do not tile / do not fit
+    assert lib.moe_i8_quant_weights(p, 7, 4, 64, 0, 0, 0, p, p, None) == abi.EUNSUPPORTED
+    assert lib.moe_i8_quant_weights(p, 0, 4, 60, 0, 0, 0, p, p, None) == abi.EINVAL
+    assert lib.moe_i8_quant_weights(p, 0, 4, 64, 3, 6, 0, p, p, None) == abi.EINVAL
+    assert lib.moe_i8_quant_weights(p, 0, 4, 64, 2, 4, 3, p, p, None) == abi.EINVAL
+    assert "row groups" in err()
+    assert lib.moe_i8_quant_weights(p, 0, 4, 64, 2, 4, 2, None, p, None) == abi.EINVAL
+    assert lib.moe_i8_quant_weights(p, 0, 0, 64, 0, 0, 0, p, p, None) == abi.OK
     # gemm: K not multiple of 64, N not multiple of 16, unknown variant, null
     base = dict(num_pairs=8, top_k=2, E=4, H=128, I=64, B=64, cap=8 + 4 * 63)
     call = lambda H=128, I=64, variant=0, x=p: lib.moe_i8_gemm_gate_up_silu(

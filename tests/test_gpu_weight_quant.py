@@ -1,0 +1,116 @@
+"""GPU parity (bit-exact): per-output-channel weight quantisation into the kernel layout through the
+C-ABI against the CPU oracle, and the quantised weights driving the layer."""
+
+import pytest
+import torch
+
+from _util import inputs_mod, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _weights(E, I, H, seed, spread=True):
+    g = torch.Generator().manual_seed(seed)
+    gate = torch.randn(E, I, H, generator=g) * H ** -0.5
+    up = torch.randn(E, I, H, generator=g) * H ** -0.5
+    down = torch.randn(E, H, I, generator=g) * I ** -0.5
+    if spread:  # row magnitudes over several decades, some rows exactly zero
+        gate *= torch.logspace(-3, 1, I)[None, :, None]
+        down[:, ::7] = 0.0
+    return gate.to(torch.bfloat16), up.to(torch.bfloat16), down.to(torch.bfloat16)
+
+
+def test_tie_vector(pra, oracle):
+    w = torch.tensor([[127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, -127.0, 3.5, 126.5, 0.0, 0.25, 0.75, -0.75, 64.5, -64.5]],
+                     dtype=torch.bfloat16)
+    q, s = pra.quantize_weights_per_channel(w.to(DEV))
+    assert q.cpu().tolist() == [[127, 0, 2, 2, 0, -2, -2, -127, 4, 126, 0, 0, 1, -1, 64, -64]]
+    assert s.cpu().tolist() == [1.0]
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 8), (5, 24), (64, 512), (33, 520), (7, 768), (16, 2048), (9, 4096),
+                                       (3, 8192), (2, 8200), (4, 16384)])
+def test_rows_match_oracle(pra, oracle, rows, cols):
+    g = torch.Generator().manual_seed(rows * 131 + cols)
+    w = (torch.randn(rows, cols, generator=g) * torch.logspace(-6, 3, rows)[:, None]).to(torch.bfloat16)
+    if rows > 2:
+        w[1] = 0.0
+        w[2] = 0.0
+        w[2, cols // 2] = 2.0 ** -100
+    q, s = pra.quantize_weights_per_channel(w.to(DEV))
+    qo, so = oracle.quantize_weights_per_channel(w)
+    assert torch.equal(q.cpu(), qo) and torch.equal(s.cpu(), so)
+
+
+@pytest.mark.parametrize("shape_name", ["toy", "qwen3-30b-a3b"])
+def test_expert_weights_layout_and_values(pra, oracle, shape_name):
+    shape = inputs_mod().SHAPES[shape_name]
+    E = min(shape.E_total, 16)
+    gate, up, down = _weights(E, shape.I, shape.H, seed=3)
+    w13, s13, w2, s2 = pra.quantize_expert_weights(gate.to(DEV), up.to(DEV), down.to(DEV))
+    o13, os13, o2, os2 = oracle.quantize_expert_weights(gate, up, down)
+    assert w13.shape == (E, 2 * shape.I, shape.H) and w2.shape == (E, shape.H, shape.I)
+    assert torch.equal(w13.cpu(), o13) and torch.equal(s13.cpu(), os13)
+    assert torch.equal(w2.cpu(), o2) and torch.equal(s2.cpu(), os2)
+
+
+def test_in_place_update_of_engine_parameters(pra, oracle):
+    # a policy step changes the trainer weights; the engine's tensors are overwritten where they lie
+    shape = inputs_mod().SHAPES["toy"]
+    E, I, H = shape.E_total, shape.I, shape.H
+    g0 = [t.to(DEV) for t in _weights(E, I, H, seed=10, spread=False)]
+    params = pra.quantize_expert_weights(*g0)
+    ptrs = [t.data_ptr() for t in params]
+    new = _weights(E, I, H, seed=11, spread=False)
+    again = pra.quantize_expert_weights(*[t.to(DEV) for t in new], out=params)
+    assert [t.data_ptr() for t in again] == ptrs
+    want = oracle.quantize_expert_weights(*new)
+    for got, ref in zip(params, want):
+        assert torch.equal(got.cpu(), ref)
+    # and the layer on the updated parameters equals the oracle's layer on the oracle's parameters
+    im = inputs_mod()
+    x = torch.randn(48, H, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16)
+    tw, ids = im.route(shape, 48, torch.Generator().manual_seed(3))
+    out = pra.fused_experts(x.to(DEV), params[0], params[2], tw.to(DEV), ids.to(DEV), use_int8_w8a8=True,
+                            per_channel_quant=True, w1_scale=params[1], w2_scale=params[3])
+    ref = oracle.fused_experts(x, want[0], want[2], tw, ids, want[1], want[3])
+    assert rel_err(out.cpu(), ref) < 1e-2
+
+
+def test_full_size_properties(pra):
+    # Qwen3-30B-A3B layer at full size (E=128): properties that need no CPU pass over 600 MB
+    shape = inputs_mod().SHAPES["qwen3-30b-a3b"]
+    E, I, H = shape.E_total, shape.I, shape.H
+    g = torch.Generator(device=DEV).manual_seed(4)
+    gate = (torch.randn(E, I, H, generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    up = (torch.randn(E, I, H, generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    down = (torch.randn(E, H, I, generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    w13, s13, w2, s2 = pra.quantize_expert_weights(gate, up, down)
+    for w, q, s in ((gate, w13[:, :I], s13[:, :I]), (up, w13[:, I:], s13[:, I:]), (down, w2, s2)):
+        wf = w.float()
+        absmax = wf.abs().amax(-1)
+        # tensor / tensor: a true division (tensor / python-float multiplies by a rounded reciprocal)
+        same_scale = torch.equal(s, (absmax / torch.full_like(absmax, 127.0)).clamp(min=1e-12))
+        assert same_scale
+        hits_127 = bool((q.abs().amax(-1) == 127).all())
+        assert hits_127
+        s64 = s.double()[..., None]
+        half_step = bool(((q.double() * s64 - wf.double()).abs() <= s64 * (0.5 + 127 * 2.0 ** -23)).all())
+        assert half_step
+    # negation symmetry and idempotence on the dequantised weights' grid
+    w13n, s13n, _, _ = pra.quantize_expert_weights(-gate, -up, down)
+    negated = torch.equal(w13n, -w13) and torch.equal(s13n, s13)
+    assert negated
+
+
+def test_argument_errors(pra):
+    w = torch.zeros(4, 16, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(NotImplementedError):
+        pra.quantize_weights_per_channel(w.float())
+    with pytest.raises(ValueError):
+        pra.quantize_weights_per_channel(torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(ValueError):
+        pra.quantize_weights_per_channel(w.cpu())
+    with pytest.raises(ValueError):
+        pra.quantize_expert_weights(w.view(1, 4, 16), w.view(1, 4, 16), w.view(1, 4, 16))
