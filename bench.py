@@ -131,6 +131,42 @@ def time_weight_requant(pkg, torch, shape, steps: int, warmup: int) -> dict:
             "layers_per_s": 1.0 / t}
 
 
+def time_router(pkg, torch, shape, M: int, steps: int, warmup: int) -> dict:
+    """The routing step in front of the layer: fp32 logits [M, E] → top-k weights and ids (and the
+    compact routed-experts record), one launch through the C-ABI with preallocated outputs, timed
+    with an event pair per launch on the launch stream."""
+    E, k = shape.E, shape.k
+    grouped = shape.routing == "grouped"
+    g = torch.Generator(device="cuda:0").manual_seed(2)
+    logits = torch.randn(M, E, generator=g, device="cuda:0")
+    bias = torch.randn(E, generator=g, device="cuda:0").mul_(0.1) if grouped else None
+    w = torch.empty(M, k, dtype=torch.float32, device="cuda:0")
+    ids = torch.empty(M, k, dtype=torch.int32, device="cuda:0")
+    record = torch.empty(M, 1, k, dtype=torch.uint8 if E <= 256 else torch.uint16, device="cuda:0")
+    lib, abi = pkg._abi.load(), pkg._abi
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        abi.check(lib.moe_i8_route_topk(
+            logits.data_ptr(), M, E, k, abi.SCORE_SIGMOID if grouped else abi.SCORE_SOFTMAX,
+            None if bias is None else bias.data_ptr(), shape.n_group if grouped else 1,
+            shape.topk_group if grouped else 1, int(grouped), 1, 1.0, w.data_ptr(), ids.data_ptr(),
+            record.data_ptr(), 1 if E <= 256 else 2, k, 0, stream))
+
+    for _ in range(warmup):
+        launch()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    torch.cuda.synchronize()
+    for a, b in pairs:
+        a.record()
+        launch()
+        b.record()
+    torch.cuda.synchronize()
+    t = sum(a.elapsed_time(b) for a, b in pairs) / steps * 1e-3
+    nbytes = M * E * 4 + M * k * (4 + 4 + record.element_size())
+    return {"M": M, "us": t * 1e6, "bytes": nbytes, "hbm_gbps": nbytes / t / 1e9}
+
+
 def cpu_baseline(oracle, torch, base, sample_m: int) -> dict:
     m = min(sample_m, base.hidden_states.shape[0])
     args = (base.hidden_states[:m], base.w1, base.w2, base.topk_weights[:m], base.topk_ids[:m],
@@ -244,6 +280,8 @@ def main() -> int:
         "sweep": sweep,
     }
     if not args.no_sweep:
+        out["router"] = [time_router(pkg, torch, pkg.inputs.SHAPES[args.shape], M, args.steps, args.warmup)
+                         for M in ms]
         out["weight_requant"] = time_weight_requant(pkg, torch, pkg.inputs.SHAPES[args.shape],
                                                     max(args.steps // 2, 1), max(args.warmup // 2, 1))
     if not args.no_cpu:

@@ -42,6 +42,11 @@ extern "C" {
 #define MOE_I8_GEMM_STREAM 1 /* weights streamed global->registers, 16-row MFMA sub-tiles (decode) */
 #define MOE_I8_GEMM_TILE 2   /* LDS-staged double-buffered tiles, 32x32x32 MFMA (prefill) */
 
+/* Router score functions (reference TokenChoiceTopKRouter.score_func). */
+#define MOE_I8_SCORE_SOFTMAX 0      /* softmax over all experts */
+#define MOE_I8_SCORE_SIGMOID 1      /* sigmoid per expert */
+#define MOE_I8_SCORE_TOPK_SOFTMAX 2 /* select on the logits, softmax over the selected k */
+
 int moe_i8_version(void);
 const char* moe_i8_last_error(void);
 
@@ -50,6 +55,29 @@ const char* moe_i8_last_error(void);
  * expert_ids needs ceil(that / B). */
 int64_t moe_i8_sorted_capacity(int64_t num_pairs, int num_experts, int block_size);
 int64_t moe_i8_align_workspace_bytes(int64_t num_pairs, int num_experts, int block_size);
+
+/*
+ * Replaces vLLM `fused_topk(hidden_states, gating_output, topk, renormalize)` (topk_softmax op,
+ * csrc/moe/topk_softmax_kernels.cu) and `grouped_topk(..., num_expert_group, topk_group,
+ * scoring_func, routed_scaling_factor, e_score_correction_bias)`
+ * (model_executor/layers/fused_moe/fused_moe.py); in-tree semantics: TokenChoiceTopKRouter.forward,
+ * src/prime_rl/trainer/models/layers/moe.py:261-307 (fp32 scores :262-269, selection-only bias
+ * :281-283, top-k :284-289, gather of unbiased scores :290, top-k softmax :292-293, route_norm with
+ * +1e-20 :302-304, route_scale :305).
+ * logits fp32 [m, num_experts] -> topk_weights fp32 [m, top_k], topk_ids int32 [m, top_k] in
+ * descending order of the selection value, equal values by ascending expert index.
+ * num_groups > 1: experts form num_groups equal contiguous groups, a group scores the sum of its two
+ * largest selection values (group_score_top2 != 0) or its largest, only the topk_groups best groups
+ * stay eligible.
+ * capture_dtype != 0 additionally writes the ids as uint8 (1) or uint16 (2) to
+ * capture[token * capture_token_stride + capture_offset + j] — the [seq_len, layers, topk] record of
+ * src/prime_rl/inference/vllm/routed_experts.py:11-33 (stride = layers * topk, offset = layer * topk).
+ */
+int moe_i8_route_topk(const float* logits, int64_t m, int num_experts, int top_k, int score_func,
+                      const float* selection_bias, int num_groups, int topk_groups, int group_score_top2,
+                      int renormalize, float route_scale, float* topk_weights, int32_t* topk_ids,
+                      void* capture, int capture_dtype, int64_t capture_token_stride,
+                      int64_t capture_offset, void* stream);
 
 /*
  * Replaces vLLM `moe_align_block_size(topk_ids, block_size, num_experts)`

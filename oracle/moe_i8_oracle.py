@@ -32,6 +32,15 @@ Pinning status (what independent evidence each function is checked against in
   brute force in numpy float32.  Parity unpinned against an int8 checkpoint producer: the
   reference tree quantises weights to FP8 only (``trainer/models/fp8.py:5-41``); the int8
   rule here is that function with qmax = 127, a whole row as the block and the integer grid.
+* ``route_topk``             pinned: element-wise brute force in Python floats (math.exp, sorted by
+  (-value, index)); closed forms (weights of the softmax router sum to 1 after renormalisation,
+  a selection bias changes which experts are chosen but not the weights of those chosen, the
+  grouped router only returns experts of ``topk_groups`` groups, one group = the ungrouped router);
+  agreement with the older ``softmax_topk`` / ``grouped_topk`` restatements.  Order among exactly
+  equal selection values is this build's rule (ascending index); ``torch.topk`` leaves it open.
+* ``serialize_routed_experts`` pinned: the two payloads of the reference's own tests
+  (``tests/unit/inference/test_serving_tokens.py:46-60``: a 2x2x2 int64 array round-trips as uint8;
+  ``"AQID"`` is bytes 1,2,3 of shape [1,1,3]) and the uint16 switch above 255.
 * ``fused_experts`` (whole)  parity unpinned at the vLLM boundary: no test or
   fixture in the reference touches int8 ``fused_experts``.  Pinned only against
   ``native_w8a8_moe`` (an independent per-expert formulation) and against the
@@ -61,6 +70,8 @@ __all__ = [
     "grouped_topk",
     "quantize_weights_per_channel",
     "quantize_expert_weights",
+    "route_topk",
+    "serialize_routed_experts",
 ]
 
 
@@ -385,3 +396,76 @@ def quantize_expert_weights(gate_proj: torch.Tensor, up_proj: torch.Tensor, down
     w13, s13 = quantize_weights_per_channel(torch.cat([gate_proj, up_proj], dim=1))
     w2, s2 = quantize_weights_per_channel(down_proj)
     return w13, s13, w2, s2
+
+
+# --------------------------------------------------------------------------- #
+# Router (restated from the reference) and the routed-experts record
+# --------------------------------------------------------------------------- #
+def route_topk(
+    logits: torch.Tensor,
+    k: int,
+    score_func: str = "softmax",
+    renormalize: bool = True,
+    route_scale: float = 1.0,
+    selection_bias: torch.Tensor | None = None,
+    num_groups: int = 1,
+    topk_groups: int = 1,
+    group_top2: bool = False,
+):
+    """``TokenChoiceTopKRouter.forward`` after the gate GEMM (``trainer/models/layers/moe.py:261-307``):
+    scores in fp32 (:262-269), bias for selection only (:281-283), top-k (:284-289), gather of the
+    unbiased scores (:290), softmax over the selected for ``topk_softmax`` (:292-293), ``route_norm``
+    with ``+1e-20`` (:302-304), ``route_scale`` (:305); plus the group pre-selection of the published
+    DeepSeek routers (group score = largest, or sum of the two largest, selection value).  Order:
+    descending selection value, equal values by ascending index (a stable sort)."""
+    lf = logits.to(torch.float32)
+    M, E = lf.shape
+    if score_func == "softmax":
+        scores = torch.softmax(lf, dim=1)
+    elif score_func == "sigmoid":
+        scores = torch.sigmoid(lf)
+    elif score_func == "topk_softmax":
+        scores = lf
+    else:
+        raise NotImplementedError(f"Unknown score function {score_func}")
+    sel = scores if selection_bias is None else scores + selection_bias.to(torch.float32).reshape(1, E)
+    if num_groups > 1:
+        per = E // num_groups
+        grouped = sel.view(M, num_groups, per)
+        gs = grouped.topk(2, dim=-1)[0].sum(dim=-1) if group_top2 else grouped.amax(dim=-1)
+        gorder = torch.sort(gs, dim=-1, descending=True, stable=True)[1][:, :topk_groups]
+        gmask = torch.zeros((M, num_groups), dtype=torch.bool).scatter_(1, gorder, True)
+        sel = sel.masked_fill(~gmask.unsqueeze(-1).expand(M, num_groups, per).reshape(M, E), float("-inf"))
+    ids = torch.sort(sel, dim=1, descending=True, stable=True)[1][:, :k]
+    w = scores.gather(1, ids)
+    if score_func == "topk_softmax":
+        w = torch.softmax(w, dim=-1)
+    if renormalize:
+        w = w / (w.sum(dim=-1, keepdim=True) + 1e-20)
+    w = w * route_scale
+    return w.to(torch.float32), ids.to(torch.int32)
+
+
+def serialize_routed_experts(routed_experts, start: int = 0):
+    """``serialize_routed_experts`` of ``inference/vllm/routed_experts.py:11-33``: a 3-d integer array
+    ``[seq_len, layers, topk]`` becomes base64 of its uint8 bytes (uint16 when an id exceeds 255)
+    with ``shape``, ``start`` and ``dtype``."""
+    import base64
+
+    if routed_experts is None:
+        return None
+    array = np.asarray(routed_experts)
+    assert array.ndim == 3 and np.issubdtype(array.dtype, np.integer)
+    dtype = np.uint8
+    if array.size:
+        assert array.min() >= 0
+        if array.max() > 255:
+            assert array.max() <= 65535
+            dtype = np.uint16
+    compact = np.ascontiguousarray(array.astype(dtype, copy=False))
+    return {
+        "data": base64.b64encode(memoryview(compact)).decode("ascii"),
+        "shape": list(compact.shape),
+        "start": start,
+        "dtype": np.dtype(dtype).name,
+    }

@@ -8,6 +8,10 @@ from . import _abi, inputs  # noqa: F401
 from .api import (  # noqa: F401
     DEFAULT_BLOCK_SIZE_M,
     fused_experts,
+    fused_topk,
+    grouped_topk,
+    route_topk,
+    routed_experts_payload,
     gemm_acc_i32,
     gemm_down,
     gemm_gate_up_silu,
@@ -28,6 +32,10 @@ __all__ = [
     "quantize_weights_per_channel",
     "quantize_expert_weights",
     "moe_sum",
+    "fused_topk",
+    "grouped_topk",
+    "route_topk",
+    "routed_experts_payload",
     "gemm_gate_up_silu",
     "gemm_down",
     "gemm_acc_i32",

@@ -7,7 +7,7 @@ built, or exports fewer symbols than the header declares, importing callers get 
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_int, c_int64, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
 from pathlib import Path
 
 PKG_DIR = Path(__file__).resolve().parent
@@ -17,6 +17,7 @@ OK = 0
 EINVAL, EWORKSPACE, ELAUNCH, EUNSUPPORTED = -1, -2, -3, -4
 DTYPE_BF16 = 0
 GEMM_AUTO, GEMM_STREAM, GEMM_TILE = 0, 1, 2
+SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_TOPK_SOFTMAX = 0, 1, 2
 MAX_EXPERTS = 1024
 
 _P = c_void_p
@@ -28,6 +29,11 @@ SIGNATURES = {
     "moe_i8_align_workspace_bytes": (c_int64, [c_int64, c_int, c_int]),
     "moe_i8_align_block_size": (c_int, [_P, c_int64, c_int, c_int, _P, c_int64, _P, c_int64, _P, _P, c_int64, _P]),
     "moe_i8_quant_rows": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, c_int, c_int64, _P, _P, _P]),
+    "moe_i8_route_topk": (
+        c_int,
+        [_P, c_int64, c_int, c_int, c_int, _P, c_int, c_int, c_int, c_int, c_float, _P, _P, _P, c_int, c_int64,
+         c_int64, _P],
+    ),
     "moe_i8_quant_weights": (c_int, [_P, c_int, c_int64, c_int64, c_int64, c_int64, c_int64, _P, _P, _P]),
     "moe_i8_gemm_gate_up_silu": (
         c_int,

@@ -23,6 +23,10 @@ __all__ = [
     "quantize_weights_per_channel",
     "quantize_expert_weights",
     "moe_sum",
+    "fused_topk",
+    "grouped_topk",
+    "route_topk",
+    "routed_experts_payload",
     "gemm_gate_up_silu",
     "gemm_down",
     "gemm_acc_i32",
@@ -259,6 +263,135 @@ def moe_sum(input: torch.Tensor, output: torch.Tensor) -> None:
 
 
 # --------------------------------------------------------------------------------------------- #
+_SCORE_FUNCS = {
+    "softmax": _abi.SCORE_SOFTMAX,
+    "sigmoid": _abi.SCORE_SIGMOID,
+    "topk_softmax": _abi.SCORE_TOPK_SOFTMAX,
+}
+
+
+def route_topk(
+    gating_output: torch.Tensor,
+    topk: int,
+    *,
+    score_func: str = "softmax",
+    renormalize: bool = True,
+    route_scale: float = 1.0,
+    selection_bias: torch.Tensor | None = None,
+    num_expert_group: int = 1,
+    topk_group: int = 1,
+    group_score_top2: bool = False,
+    routed_experts_out: tuple[torch.Tensor, int] | None = None,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """The reference router after its gate GEMM (``TokenChoiceTopKRouter.forward``,
+    ``src/prime_rl/trainer/models/layers/moe.py:261-307``) in one launch: fp32 scores
+    (``score_func`` ∈ softmax / sigmoid / topk_softmax), a bias that only steers the selection,
+    optional group pre-selection, top-k in descending order (equal values by ascending index),
+    ``route_norm`` (``renormalize``: divide by sum + 1e-20) and ``route_scale``.
+
+    ``gating_output`` fp32 ``[M, E]`` → ``(topk_weights fp32 [M, topk], topk_ids int32 [M, topk])``.
+    ``routed_experts_out=(record, layer)`` also writes the ids into ``record[:, layer, :]`` of a
+    uint8 / uint16 ``[M, layers, topk]`` tensor, the compact routed-experts record of
+    ``src/prime_rl/inference/vllm/routed_experts.py:11-33``.
+    """
+    _require_gpu("gating_output", gating_output)
+    if gating_output.dtype != torch.float32:
+        raise NotImplementedError(f"router logits must be float32, got {gating_output.dtype}")
+    if gating_output.dim() != 2:
+        raise ValueError("gating_output must be [M, E]")
+    if score_func not in _SCORE_FUNCS:
+        raise NotImplementedError(f"Unknown score function {score_func}")
+    M, E = gating_output.shape
+    if selection_bias is not None:
+        _require_gpu("selection_bias", selection_bias)
+        if selection_bias.dtype != torch.float32 or selection_bias.numel() != E:
+            raise ValueError("selection_bias must be float32 with one element per expert")
+    capture, capture_dtype, stride, offset = None, 0, 0, 0
+    if routed_experts_out is not None:
+        record, layer = routed_experts_out
+        _require_gpu("routed_experts_out[0]", record)
+        if record.dtype not in (torch.uint8, torch.uint16):
+            raise ValueError("the routed-experts record must be uint8 or uint16")
+        if record.dim() != 3 or record.shape[0] != M or record.shape[2] != topk:
+            raise ValueError(f"the routed-experts record must be [M, layers, topk] = [{M}, *, {topk}]")
+        if not 0 <= layer < record.shape[1]:
+            raise ValueError("layer index outside the routed-experts record")
+        capture, capture_dtype = record, 1 if record.dtype == torch.uint8 else 2
+        stride, offset = record.shape[1] * topk, layer * topk
+    weights = torch.empty((M, topk), dtype=torch.float32, device=gating_output.device)
+    ids = torch.empty((M, topk), dtype=torch.int32, device=gating_output.device)
+    _abi.check(
+        _abi.load().moe_i8_route_topk(
+            _ptr(gating_output), M, E, topk, _SCORE_FUNCS[score_func], _ptr(selection_bias), num_expert_group,
+            topk_group, int(group_score_top2), int(renormalize), float(route_scale), _ptr(weights), _ptr(ids),
+            _ptr(capture), capture_dtype, stride, offset, _stream(gating_output),
+        )
+    )
+    return weights, ids
+
+
+def fused_topk(
+    hidden_states: torch.Tensor,
+    gating_output: torch.Tensor,
+    topk: int,
+    renormalize: bool,
+    *,
+    routed_experts_out: tuple[torch.Tensor, int] | None = None,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """vLLM ``fused_topk``: softmax over all experts, top-k, optional renormalisation.
+    ``hidden_states`` is only checked for its token count, as upstream."""
+    if hidden_states.shape[0] != gating_output.shape[0]:
+        raise ValueError("Number of tokens mismatch")
+    return route_topk(gating_output, topk, score_func="softmax", renormalize=renormalize,
+                      routed_experts_out=routed_experts_out)
+
+
+def grouped_topk(
+    hidden_states: torch.Tensor,
+    gating_output: torch.Tensor,
+    topk: int,
+    renormalize: bool,
+    num_expert_group: int = 0,
+    topk_group: int = 0,
+    scoring_func: str = "softmax",
+    routed_scaling_factor: float = 1.0,
+    e_score_correction_bias: torch.Tensor | None = None,
+    *,
+    routed_experts_out: tuple[torch.Tensor, int] | None = None,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """vLLM ``grouped_topk`` (DeepSeek-style): with a correction bias a group scores the sum of its
+    two largest biased scores, without one its largest score; the ``topk_group`` best of
+    ``num_expert_group`` groups stay eligible; weights are the unbiased scores."""
+    if hidden_states.shape[0] != gating_output.shape[0]:
+        raise ValueError("Number of tokens mismatch")
+    if scoring_func not in ("softmax", "sigmoid"):
+        raise ValueError(f"Unsupported scoring function: {scoring_func}")
+    return route_topk(
+        gating_output, topk, score_func=scoring_func, renormalize=renormalize, route_scale=routed_scaling_factor,
+        selection_bias=e_score_correction_bias, num_expert_group=max(num_expert_group, 1),
+        topk_group=max(topk_group, 1), group_score_top2=e_score_correction_bias is not None,
+        routed_experts_out=routed_experts_out,
+    )
+
+
+def routed_experts_payload(record: torch.Tensor, start: int = 0) -> dict:
+    """The wire form of a routed-experts record ``[seq_len, layers, topk]`` (uint8 / uint16), field
+    for field what ``serialize_routed_experts`` builds
+    (``src/prime_rl/inference/vllm/routed_experts.py:27-33``): base64 of the raw bytes, shape, start
+    and dtype name.  The record is already compact on the GPU, so this is one copy to the host."""
+    import base64
+
+    if record.dim() != 3 or record.dtype not in (torch.uint8, torch.uint16):
+        raise ValueError("record must be a uint8 or uint16 [seq_len, layers, topk] tensor")
+    host = record.contiguous().cpu().numpy()
+    return {
+        "data": base64.b64encode(memoryview(host)).decode("ascii"),
+        "shape": list(host.shape),
+        "start": start,
+        "dtype": host.dtype.name,
+    }
+
+
 def _check_routing(sorted_token_ids, expert_ids, num_tokens_post_padded):
     for name, t in (
         ("sorted_token_ids", sorted_token_ids),

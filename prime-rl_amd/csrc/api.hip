@@ -150,6 +150,59 @@ int moe_i8_quant_rows(const void* x, int dtype, int64_t src_rows, int64_t cols, 
   return check_launch(moe_i8::launch_quant_rows(a, static_cast<hipStream_t>(stream)), "quant_rows");
 }
 
+int moe_i8_route_topk(const float* logits, int64_t m, int num_experts, int top_k, int score_func,
+                      const float* selection_bias, int num_groups, int topk_groups, int group_score_top2,
+                      int renormalize, float route_scale, float* topk_weights, int32_t* topk_ids,
+                      void* capture, int capture_dtype, int64_t capture_token_stride,
+                      int64_t capture_offset, void* stream) {
+  if (m < 0) return fail(MOE_I8_EINVAL, "negative token count");
+  if (num_experts < 1 || num_experts > MOE_I8_MAX_EXPERTS)
+    return fail(MOE_I8_EINVAL, "num_experts (%d) must be in [1, %d]", num_experts, MOE_I8_MAX_EXPERTS);
+  if (top_k < 1 || top_k > num_experts || top_k > 64)
+    return fail(MOE_I8_EINVAL, "top_k (%d) must be in [1, min(num_experts, 64)]", top_k);
+  if (score_func != MOE_I8_SCORE_SOFTMAX && score_func != MOE_I8_SCORE_SIGMOID &&
+      score_func != MOE_I8_SCORE_TOPK_SOFTMAX)
+    return fail(MOE_I8_EINVAL, "unknown score function %d", score_func);
+  if (num_groups < 1 || num_experts % num_groups) return fail(MOE_I8_EINVAL, "num_groups must divide num_experts");
+  if (num_groups > 1) {
+    const int per_lane = moe_i8::route_experts_per_lane(num_experts);
+    const int group_size = num_experts / num_groups;
+    const int lanes = group_size / per_lane;
+    if (group_size % per_lane || lanes < 1 || (lanes & (lanes - 1)))
+      return fail(MOE_I8_EUNSUPPORTED, "group size %d must be a power-of-two multiple of %d experts", group_size,
+                  per_lane);
+    if (topk_groups < 1 || topk_groups > num_groups) return fail(MOE_I8_EINVAL, "topk_groups out of range");
+    if (group_score_top2 && group_size < 2) return fail(MOE_I8_EINVAL, "top-2 group score needs groups of >= 2");
+    if (top_k > topk_groups * group_size) return fail(MOE_I8_EINVAL, "top_k exceeds the experts of the kept groups");
+  }
+  if (capture_dtype < 0 || capture_dtype > 2) return fail(MOE_I8_EINVAL, "capture dtype must be 0, 1 (u8) or 2 (u16)");
+  if (capture_dtype == 1 && num_experts > 256) return fail(MOE_I8_EINVAL, "uint8 capture holds at most 256 experts");
+  if (capture_dtype && (!capture || capture_token_stride < top_k || capture_offset < 0 ||
+                        capture_offset + top_k > capture_token_stride))
+    return fail(MOE_I8_EINVAL, "capture needs a buffer and offset + top_k <= token stride");
+  if (m == 0) return MOE_I8_OK;
+  if (!logits || !topk_weights || !topk_ids) return fail(MOE_I8_EINVAL, "null pointer");
+  moe_i8::RouteArgs a;
+  a.logits = logits;
+  a.m = m;
+  a.num_experts = num_experts;
+  a.top_k = top_k;
+  a.score_func = score_func;
+  a.bias = selection_bias;
+  a.num_groups = num_groups;
+  a.topk_groups = topk_groups;
+  a.group_top2 = group_score_top2;
+  a.renormalize = renormalize;
+  a.route_scale = route_scale;
+  a.weights = topk_weights;
+  a.ids = topk_ids;
+  a.capture = capture_dtype ? capture : nullptr;
+  a.capture_bytes = capture_dtype;
+  a.capture_stride = capture_token_stride;
+  a.capture_offset = capture_offset;
+  return check_launch(moe_i8::launch_route_topk(a, static_cast<hipStream_t>(stream)), "route_topk");
+}
+
 int moe_i8_quant_weights(const void* w, int dtype, int64_t rows, int64_t cols, int64_t rows_per_group,
                          int64_t out_rows_per_group, int64_t out_row_offset, int8_t* q, float* scale,
                          void* stream) {

@@ -28,6 +28,36 @@ __device__ __forceinline__ float round_to_bf16(float f) {
   return bf16_bits_to_f32(f32_to_bf16_bits(f));
 }
 
+// Wave-wide reductions on the VALU's data-parallel-primitive lane permutes (no LDS traffic, a few
+// cycles per step): quads, half rows and rows of 16 by mirror permutes, then row 15 -> next row and
+// row 31 -> upper half broadcasts leave the total in lane 63, which is read back as a scalar.
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), kCtrl, kRowMask, 0xf, false));
+}
+__device__ __forceinline__ float wave_reduce_max(float v) {
+  v = fmaxf(v, dpp_move<0xb1, 0xf>(v));   // quad_perm [1,0,3,2]
+  v = fmaxf(v, dpp_move<0x4e, 0xf>(v));   // quad_perm [2,3,0,1]
+  v = fmaxf(v, dpp_move<0x141, 0xf>(v));  // row_half_mirror
+  v = fmaxf(v, dpp_move<0x140, 0xf>(v));  // row_mirror
+  v = fmaxf(v, dpp_move<0x142, 0xa>(v));  // row_bcast:15 into rows 1 and 3
+  v = fmaxf(v, dpp_move<0x143, 0xc>(v));  // row_bcast:31 into rows 2 and 3
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+__device__ __forceinline__ float wave_reduce_sum(float v) {
+  v += dpp_move<0xb1, 0xf>(v);
+  v += dpp_move<0x4e, 0xf>(v);
+  v += dpp_move<0x141, 0xf>(v);
+  v += dpp_move<0x140, 0xf>(v);
+  // the broadcasts must add only into the rows they target: elsewhere the permute returns the
+  // lane's own value and would double it
+  const float b15 = dpp_move<0x142, 0xa>(v);
+  v += (lane_id() & 16) ? b15 : 0.0f;
+  const float b31 = dpp_move<0x143, 0xc>(v);
+  v += (lane_id() & 32) ? b31 : 0.0f;
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
 typedef float f2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
 
@@ -103,6 +133,30 @@ struct QuantArgs {
   int64_t out_row_offset = 0;
 };
 hipError_t launch_quant_rows(const QuantArgs& a, hipStream_t stream);
+// Router: scores -> (grouped) top-k -> weights, one wavefront per token.
+enum ScoreFunc { kScoreSoftmax = 0, kScoreSigmoid = 1, kScoreTopkSoftmax = 2 };
+struct RouteArgs {
+  const float* logits;  // [m, num_experts]
+  int64_t m;
+  int num_experts;
+  int top_k;
+  int score_func;
+  const float* bias;  // [num_experts] or null; added for selection only
+  int num_groups;     // 1 = no group pre-selection
+  int topk_groups;
+  int group_top2;  // group score: 1 = sum of the two largest selection values, 0 = the largest
+  int renormalize;
+  float route_scale;
+  float* weights;  // [m, top_k]
+  int32_t* ids;    // [m, top_k]
+  void* capture;   // compact copy of ids at capture[tok * capture_stride + capture_offset + j]
+  int capture_bytes;  // 0 = none, 1 = uint8, 2 = uint16
+  int64_t capture_stride;
+  int64_t capture_offset;
+};
+int route_experts_per_lane(int num_experts);
+hipError_t launch_route_topk(const RouteArgs& a, hipStream_t stream);
+
 // Per-output-channel weight quantisation (round to nearest even of w / scale, scale = absmax / 127).
 hipError_t launch_quant_weights(const QuantArgs& a, hipStream_t stream);
 // moe_align and the quantisation of `q` in one launch; only when align_quant_fusable() says so.

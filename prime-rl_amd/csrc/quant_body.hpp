@@ -8,11 +8,7 @@ namespace moe_i8 {
 
 constexpr int kQuantVec = 8;  // bf16 elements per 16-byte load
 
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int d = kWave / 2; d >= 1; d >>= 1) v = fmaxf(v, __shfl_xor(v, d));
-  return v;
-}
+__device__ __forceinline__ float wave_max(float v) { return wave_reduce_max(v); }
 
 __device__ __forceinline__ float absmax8(const uint4& v) {
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};

@@ -63,6 +63,15 @@ def test_c_abi_rejects_bad_arguments_without_launching(pra):
     assert lib.moe_i8_quant_rows(p, 0, 4, 64, 32, None, 1, 4, p, p, None) == abi.EINVAL
     assert lib.moe_i8_quant_rows(None, 0, 4, 64, 64, None, 1, 4, p, p, None) == abi.EINVAL
     assert lib.moe_i8_quant_rows(p, 0, 4, 64, 64, None, 1, 0, p, p, None) == abi.OK  # zero rows: no-op
+    # router: expert / top-k limits, groups that do not tile, capture that does not fit
+    rt = lambda E=128, k=8, score=0, G=1, KG=1, cap=None, cdt=0, stride=0, off=0: lib.moe_i8_route_topk(
+        p, 4, E, k, score, None, G, KG, 0, 1, 1.0, p, p, cap, cdt, stride, off, None)
+    assert rt(E=2000) == abi.EINVAL and rt(k=0) == abi.EINVAL and rt(k=65, E=128) == abi.EINVAL
+    assert rt(score=5) == abi.EINVAL and rt(G=3) == abi.EINVAL
+    assert rt(E=192, G=4, KG=1) == abi.EUNSUPPORTED  # 48-expert groups = 12 lanes of 4: not a power of two
+    assert rt(G=8, KG=9) == abi.EINVAL and rt(G=8, KG=1, k=17) == abi.EINVAL
+    assert rt(E=512, cap=p, cdt=1, stride=8) == abi.EINVAL and "uint8" in err()
+    assert rt(cap=p, cdt=1, stride=8, off=1) == abi.EINVAL and rt(cap=None, cdt=2, stride=8) == abi.EINVAL
     # weight quant: dtype, cols, row groups that do not tile / do not fit
     assert lib.moe_i8_quant_weights(p, 7, 4, 64, 0, 0, 0, p, p, None) == abi.EUNSUPPORTED
     assert lib.moe_i8_quant_weights(p, 0, 4, 60, 0, 0, 0, p, p, None) == abi.EINVAL
