@@ -167,6 +167,26 @@ def time_router(pkg, torch, shape, M: int, steps: int, warmup: int) -> dict:
     return {"M": M, "us": t * 1e6, "bytes": nbytes, "hbm_gbps": nbytes / t / 1e9}
 
 
+def time_dense_mlp(pkg, torch, M: int, H: int, I: int, steps: int, warmup: int) -> dict:
+    """The shared-expert / dense W8A8 gated MLP on the same GEMM kernels with one group."""
+    g = torch.Generator(device="cuda:0").manual_seed(3)
+    x = torch.randn(M, H, generator=g, device="cuda:0").to(torch.bfloat16)
+    w13 = torch.randint(-127, 128, (2 * I, H), generator=g, dtype=torch.int8, device="cuda:0")
+    w2 = torch.randint(-127, 128, (H, I), generator=g, dtype=torch.int8, device="cuda:0")
+    s13 = torch.rand(2 * I, generator=g, device="cuda:0") * 0.002 + 0.001
+    s2 = torch.rand(H, generator=g, device="cuda:0") * 0.002 + 0.001
+    for _ in range(warmup):
+        pkg.w8a8_mlp(x, w13, s13, w2, s2)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        pkg.w8a8_mlp(x, w13, s13, w2, s2)
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / steps
+    ops = 6 * M * I * H
+    return {"M": M, "H": H, "I": I, "us": t * 1e6, "int8_tops": ops / t / 1e12, "mfma_frac": ops / t / PEAK_INT8_OPS}
+
+
 def cpu_baseline(oracle, torch, base, sample_m: int) -> dict:
     m = min(sample_m, base.hidden_states.shape[0])
     args = (base.hidden_states[:m], base.w1, base.w2, base.topk_weights[:m], base.topk_ids[:m],
@@ -282,6 +302,9 @@ def main() -> int:
     if not args.no_sweep:
         out["router"] = [time_router(pkg, torch, pkg.inputs.SHAPES[args.shape], M, args.steps, args.warmup)
                          for M in ms]
+        shape_h = pkg.inputs.SHAPES[args.shape]
+        out["dense_mlp"] = [time_dense_mlp(pkg, torch, M, shape_h.H, shape_h.I, args.steps, args.warmup)
+                            for M in (args.m, 8 * args.m)]
         out["weight_requant"] = time_weight_requant(pkg, torch, pkg.inputs.SHAPES[args.shape],
                                                     max(args.steps // 2, 1), max(args.warmup // 2, 1))
     if not args.no_cpu:

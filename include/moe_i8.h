@@ -141,7 +141,7 @@ int moe_i8_gemm_gate_up_silu(const int8_t* x_q, const float* a_scale, const int8
  * In-tree semantics: weight applied after the experts in fp32 then cast,
  * trainer/distributed/token_dispatcher.py:159-160.
  * h_q int8 [num_pairs, I], a_scale fp32 [num_pairs], w2 int8 [E, H, I],
- * w2_scale fp32 [E, H], topk_weights fp32 [num_pairs] -> out bf16 [num_pairs, H].
+ * w2_scale fp32 [E, H], topk_weights fp32 [num_pairs] (NULL = all ones) -> out bf16 [num_pairs, H].
  */
 int moe_i8_gemm_down(const int8_t* h_q, const float* a_scale, const int8_t* w2,
                      const float* w2_scale, const float* topk_weights,
@@ -185,6 +185,31 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
                          const float* w1_scale, const float* w2_scale, void* out, int64_t m,
                          int top_k, int num_experts, int hidden_size, int inter, int block_size,
                          void* workspace, int64_t workspace_bytes, int variant, void* stream);
+
+/*
+ * Dense W8A8 layers (shared experts, dense first-k MLPs) on the same kernels with one group.
+ *
+ * moe_i8_scaled_int8_quant replaces vLLM `ops.scaled_int8_quant(x, scale=None)` (dynamic per-token
+ * symmetric, csrc/quantization/compressed_tensors/int8_quant_kernels.cu): q = rint(x * (127 / absmax)),
+ * ties to even — the rounding that separates it from per_token_quant_int8 above; scale = absmax / 127.
+ *
+ * moe_i8_w8a8_linear replaces `ops.cutlass_scaled_mm(x_q, w.t(), scale_a, scale_b, out_dtype=bf16)` after
+ * that quantisation: x bf16 [m, k], w int8 [n, k], w_scale fp32 [n] -> out bf16 [m, n] =
+ * bf16((acc * a_scale) * w_scale).
+ *
+ * moe_i8_w8a8_mlp is the shared-expert MLP down(silu(gate(x)) * up(x))
+ * (FeedForward.forward, src/prime_rl/trainer/models/layers/mlp.py:29-32; added to the routed output at
+ * src/prime_rl/trainer/models/layers/moe.py:453-462): w13 int8 [2*inter, hidden] gate rows first,
+ * w2 int8 [hidden, inter]; x bf16 [m, hidden] -> out bf16 [m, hidden].
+ */
+int moe_i8_scaled_int8_quant(const void* x, int dtype, int64_t rows, int64_t cols, int64_t row_stride,
+                             int8_t* q, float* scale, void* stream);
+int64_t moe_i8_dense_workspace_bytes(int64_t m, int k, int inter /* 0 for the plain linear */);
+int moe_i8_w8a8_linear(const void* x, const int8_t* w, const float* w_scale, void* out, int64_t m, int n,
+                       int k, void* workspace, int64_t workspace_bytes, int variant, void* stream);
+int moe_i8_w8a8_mlp(const void* x, const int8_t* w13, const float* w13_scale, const int8_t* w2,
+                    const float* w2_scale, void* out, int64_t m, int hidden, int inter, void* workspace,
+                    int64_t workspace_bytes, int variant, void* stream);
 
 #ifdef __cplusplus
 }

@@ -41,6 +41,11 @@ Pinning status (what independent evidence each function is checked against in
 * ``serialize_routed_experts`` pinned: the two payloads of the reference's own tests
   (``tests/unit/inference/test_serving_tokens.py:46-60``: a 2x2x2 int64 array round-trips as uint8;
   ``"AQID"`` is bytes 1,2,3 of shape [1,1,3]) and the uint16 switch above 255.
+* ``scaled_int8_quant`` / ``w8a8_linear`` / ``w8a8_mlp``  pinned: tie vector (even, and different from the
+  half-away quantiser on it), numpy float32 brute force; the linear against a float64 matmul of the
+  dequantised operands; the MLP against the MoE layer with one expert that every token visits (which
+  differs only in the rounding of ties) and against the fp32 MLP.  Parity unpinned at the vLLM
+  boundary (``scaled_int8_quant`` / ``cutlass_scaled_mm`` are not in the reference tree).
 * ``fused_experts`` (whole)  parity unpinned at the vLLM boundary: no test or
   fixture in the reference touches int8 ``fused_experts``.  Pinned only against
   ``native_w8a8_moe`` (an independent per-expert formulation) and against the
@@ -72,6 +77,9 @@ __all__ = [
     "quantize_expert_weights",
     "route_topk",
     "serialize_routed_experts",
+    "scaled_int8_quant",
+    "w8a8_linear",
+    "w8a8_mlp",
 ]
 
 
@@ -469,3 +477,30 @@ def serialize_routed_experts(routed_experts, start: int = 0):
         "start": start,
         "dtype": np.dtype(dtype).name,
     }
+
+
+# --------------------------------------------------------------------------- #
+# Dense W8A8 (shared experts, dense MLPs)
+# --------------------------------------------------------------------------- #
+def scaled_int8_quant(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """vLLM ``scaled_int8_quant`` (dynamic, per token, symmetric): as ``per_token_quant_int8`` but the
+    product ``x * (127 / absmax)`` is rounded to nearest with ties to even."""
+    xf = x.to(torch.float32)
+    absmax = xf.abs().amax(dim=-1, keepdim=True).clamp_min(1e-10)
+    inv = torch.full_like(absmax, 127.0) / absmax
+    return torch.round(xf * inv).to(torch.int8), absmax / 127.0
+
+
+def w8a8_linear(x: torch.Tensor, w: torch.Tensor, w_scale: torch.Tensor) -> torch.Tensor:
+    """``bf16((acc * a_scale) * w_scale)`` with ``acc = x_q @ w.T`` in int32; ``w`` int8 ``[N, K]``."""
+    q, a = scaled_int8_quant(x.reshape(-1, x.shape[-1]))
+    acc = _int_mm(q, w).to(torch.float32)
+    out = ((acc * a) * w_scale.reshape(1, -1)).to(torch.bfloat16)
+    return out.reshape(*x.shape[:-1], w.shape[0])
+
+
+def w8a8_mlp(x, w13, w13_scale, w2, w2_scale) -> torch.Tensor:
+    """``down(silu(gate(x)) * up(x))`` (``trainer/models/layers/mlp.py:29-32``) with both linears W8A8 and the
+    activation evaluated on bf16 values as ``silu_and_mul`` does."""
+    c = w8a8_linear(x, w13, w13_scale)
+    return w8a8_linear(silu_and_mul(c), w2, w2_scale)

@@ -7,11 +7,14 @@ The directory name carries a hyphen, so import it through the top-level ``prime_
 from . import _abi, inputs  # noqa: F401
 from .api import (  # noqa: F401
     DEFAULT_BLOCK_SIZE_M,
+    apply_int8_linear,
     fused_experts,
     fused_topk,
     grouped_topk,
     route_topk,
     routed_experts_payload,
+    scaled_int8_quant,
+    w8a8_mlp,
     gemm_acc_i32,
     gemm_down,
     gemm_gate_up_silu,
@@ -36,6 +39,9 @@ __all__ = [
     "grouped_topk",
     "route_topk",
     "routed_experts_payload",
+    "scaled_int8_quant",
+    "apply_int8_linear",
+    "w8a8_mlp",
     "gemm_gate_up_silu",
     "gemm_down",
     "gemm_acc_i32",

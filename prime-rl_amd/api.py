@@ -27,6 +27,9 @@ __all__ = [
     "grouped_topk",
     "route_topk",
     "routed_experts_payload",
+    "scaled_int8_quant",
+    "apply_int8_linear",
+    "w8a8_mlp",
     "gemm_gate_up_silu",
     "gemm_down",
     "gemm_acc_i32",
@@ -390,6 +393,117 @@ def routed_experts_payload(record: torch.Tensor, start: int = 0) -> dict:
         "start": start,
         "dtype": host.dtype.name,
     }
+
+
+def scaled_int8_quant(
+    input: torch.Tensor, scale: torch.Tensor | None = None, azp: torch.Tensor | None = None, symmetric: bool = True
+) -> tuple[torch.Tensor, torch.Tensor, None]:
+    """vLLM ``ops.scaled_int8_quant`` in its dynamic per-token symmetric form: ``(q int8 like input,
+    scales fp32 [..., 1], None)``, ``q = rint(x * (127 / absmax))`` with ties to even (the dense-layer
+    quantiser; ``per_token_quant_int8`` of the MoE path rounds ties away from zero)."""
+    if scale is not None or azp is not None or not symmetric:
+        raise NotImplementedError("only dynamic per-token symmetric quantisation is supported")
+    _require_gpu("input", input)
+    if input.dtype != torch.bfloat16:
+        raise NotImplementedError(f"only bfloat16 activations are supported, got {input.dtype}")
+    cols = input.shape[-1]
+    if cols % 8 or cols == 0:
+        raise ValueError("last dimension must be a positive multiple of 8")
+    rows = input.numel() // cols
+    q = torch.empty(input.shape, dtype=torch.int8, device=input.device)
+    scales = torch.empty((*input.shape[:-1], 1), dtype=torch.float32, device=input.device)
+    _abi.check(
+        _abi.load().moe_i8_scaled_int8_quant(_ptr(input), _abi.DTYPE_BF16, rows, cols, cols, _ptr(q), _ptr(scales),
+                                             _stream(input))
+    )
+    return q, scales, None
+
+
+def _dense_weight(name: str, w: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """Accept the weight as [N, K] contiguous or as vLLM holds it for scaled_mm, the [K, N] transposed view."""
+    if not isinstance(w, torch.Tensor) or not w.is_cuda:
+        raise ValueError(f"{name} must be a GPU tensor (this path has no CPU implementation)")
+    if w.dtype != torch.int8 or w.dim() != 2:
+        raise ValueError(f"{name} must be a 2-d int8 tensor")
+    if not w.is_contiguous():
+        if not w.t().is_contiguous():
+            raise ValueError(f"{name} must be [N, K] contiguous or the transposed view of such a tensor")
+        w = w.t()
+    _require_gpu(f"{name}_scale", scale)
+    if scale.dtype != torch.float32 or scale.numel() != w.shape[0]:
+        raise ValueError(f"{name}_scale must be float32 with one element per output channel")
+    return w
+
+
+def _dense_workspace(x: torch.Tensor, k: int, inter: int) -> torch.Tensor:
+    m = x.numel() // k
+    return _workspace(x.device, _stream(x), _abi.load().moe_i8_dense_workspace_bytes(m, k, inter))
+
+
+def apply_int8_linear(
+    input: torch.Tensor,
+    weight: torch.Tensor,
+    weight_scale: torch.Tensor,
+    input_scale: torch.Tensor | None = None,
+    input_zero_point: torch.Tensor | None = None,
+    azp_adj: torch.Tensor | None = None,
+    bias: torch.Tensor | None = None,
+    *,
+    gemm_variant: str | int = "auto",
+) -> torch.Tensor:
+    """vLLM's dense W8A8 int8 linear (dynamic per-token symmetric activations, per-channel weights):
+    ``scaled_int8_quant`` then ``cutlass_scaled_mm``; ``out = bf16((acc * a_scale) * w_scale)``.
+    ``weight`` int8 is ``[N, K]`` contiguous or its ``[K, N]`` transposed view."""
+    if input_scale is not None or input_zero_point is not None or azp_adj is not None:
+        raise NotImplementedError("static or asymmetric activation quantisation is not supported")
+    if bias is not None:
+        raise NotImplementedError("bias is not supported")
+    _require_gpu("input", input)
+    if input.dtype != torch.bfloat16:
+        raise NotImplementedError(f"only bfloat16 activations are supported, got {input.dtype}")
+    w = _dense_weight("weight", weight, weight_scale)
+    n, k = w.shape
+    if input.shape[-1] != k:
+        raise ValueError(f"input has {input.shape[-1]} features, weight expects {k}")
+    m = input.numel() // k
+    out = torch.empty((*input.shape[:-1], n), dtype=torch.bfloat16, device=input.device)
+    ws = _dense_workspace(input, k, 0)
+    _abi.check(
+        _abi.load().moe_i8_w8a8_linear(_ptr(input), _ptr(w), _ptr(weight_scale), _ptr(out), m, n, k, _ptr(ws),
+                                       ws.numel(), _variant(gemm_variant), _stream(input))
+    )
+    return out
+
+
+def w8a8_mlp(
+    x: torch.Tensor,
+    w13: torch.Tensor,
+    w13_scale: torch.Tensor,
+    w2: torch.Tensor,
+    w2_scale: torch.Tensor,
+    *,
+    gemm_variant: str | int = "auto",
+) -> torch.Tensor:
+    """Dense gated MLP ``down(silu(gate(x)) * up(x))`` in W8A8 (the shared expert the reference adds to the
+    routed output, ``src/prime_rl/trainer/models/layers/moe.py:453-462``; ``FeedForward.forward``,
+    ``src/prime_rl/trainer/models/layers/mlp.py:29-32``): ``w13`` int8 ``[2I, H]`` gate rows first, ``w2``
+    int8 ``[H, I]``, per-channel scales; both activations quantised per token with ties to even."""
+    _require_gpu("x", x)
+    if x.dtype != torch.bfloat16:
+        raise NotImplementedError(f"only bfloat16 activations are supported, got {x.dtype}")
+    w13 = _dense_weight("w13", w13, w13_scale)
+    w2 = _dense_weight("w2", w2, w2_scale)
+    two_i, h = w13.shape
+    if two_i % 2 or w2.shape != (h, two_i // 2) or x.shape[-1] != h:
+        raise ValueError("expected x [*, H], w13 [2I, H], w2 [H, I]")
+    m = x.numel() // h
+    out = torch.empty_like(x)
+    ws = _dense_workspace(x, h, two_i // 2)
+    _abi.check(
+        _abi.load().moe_i8_w8a8_mlp(_ptr(x), _ptr(w13), _ptr(w13_scale), _ptr(w2), _ptr(w2_scale), _ptr(out), m, h,
+                                    two_i // 2, _ptr(ws), ws.numel(), _variant(gemm_variant), _stream(x))
+    )
+    return out
 
 
 def _check_routing(sorted_token_ids, expert_ids, num_tokens_post_padded):

@@ -124,9 +124,9 @@ int moe_i8_align_block_size(const int32_t* topk_ids, int64_t num_pairs, int num_
   return check_launch(moe_i8::launch_align(a, static_cast<hipStream_t>(stream)), "moe_align");
 }
 
-int moe_i8_quant_rows(const void* x, int dtype, int64_t src_rows, int64_t cols, int64_t row_stride,
-                      const int32_t* gather, int gather_div, int64_t rows, int8_t* q, float* scale,
-                      void* stream) {
+static int quant_rows_impl(const void* x, int dtype, int64_t src_rows, int64_t cols, int64_t row_stride,
+                           const int32_t* gather, int gather_div, int64_t rows, int8_t* q, float* scale,
+                           int round_even, void* stream) {
   if (dtype != MOE_I8_DTYPE_BF16) return fail(MOE_I8_EUNSUPPORTED, "only bf16 activations are supported");
   if (rows < 0 || src_rows < 0) return fail(MOE_I8_EINVAL, "negative row count");
   if (rows == 0) return MOE_I8_OK;
@@ -147,7 +147,19 @@ int moe_i8_quant_rows(const void* x, int dtype, int64_t src_rows, int64_t cols, 
   a.rows = rows;
   a.q = q;
   a.scale = scale;
+  a.round_even = round_even;
   return check_launch(moe_i8::launch_quant_rows(a, static_cast<hipStream_t>(stream)), "quant_rows");
+}
+
+int moe_i8_quant_rows(const void* x, int dtype, int64_t src_rows, int64_t cols, int64_t row_stride,
+                      const int32_t* gather, int gather_div, int64_t rows, int8_t* q, float* scale,
+                      void* stream) {
+  return quant_rows_impl(x, dtype, src_rows, cols, row_stride, gather, gather_div, rows, q, scale, 0, stream);
+}
+
+int moe_i8_scaled_int8_quant(const void* x, int dtype, int64_t rows, int64_t cols, int64_t row_stride,
+                             int8_t* q, float* scale, void* stream) {
+  return quant_rows_impl(x, dtype, rows, cols, row_stride, nullptr, 1, rows, q, scale, 1, stream);
 }
 
 int moe_i8_route_topk(const float* logits, int64_t m, int num_experts, int top_k, int score_func,
@@ -280,7 +292,7 @@ int moe_i8_gemm_down(const int8_t* h_q, const float* a_scale, const int8_t* w2,
                                  num_pairs, num_experts, hidden, inter, block_size, sorted_cap,
                                  variant))
     return rc;
-  if (!a_scale || !w2_scale || !topk_weights) return fail(MOE_I8_EINVAL, "null scale pointer");
+  if (!a_scale || !w2_scale) return fail(MOE_I8_EINVAL, "null scale pointer");
   if (!aligned16(w2_scale)) return fail(MOE_I8_EINVAL, "w2_scale must be 16-byte aligned");
   moe_i8::GemmArgs g{};
   g.mode = moe_i8::kDown;
@@ -459,6 +471,99 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
                                 hidden_size, inter, block_size, c.cap, down, variant, stream))
     return rc;
   return moe_i8_sum(down, out, m, top_k, hidden_size, stream);
+}
+
+// Workspace of the dense entry points (every region 256-byte aligned):
+//   x_q i8[M*K] | a1 f32[M] | sorted i32[cap] | expert_ids i32[cap/64] | npp i32[1] |
+//   (mlp only) act bf16[M*I] | act_q i8[M*I] | a2 f32[M]
+namespace {
+constexpr int kDenseBlock = 64;
+struct DenseCarve {
+  int64_t x_q, a1, sorted, eids, npp, act, act_q, a2, total, cap;
+};
+DenseCarve dense_carve(int64_t m, int k, int inter) {
+  DenseCarve c{};
+  c.cap = moe_i8_sorted_capacity(m, 1, kDenseBlock);
+  int64_t off = 0;
+  auto take = [&](int64_t bytes) {
+    const int64_t at = off;
+    off = align_up(off + bytes, 256);
+    return at;
+  };
+  c.x_q = take(m * k);
+  c.a1 = take(m * 4);
+  c.sorted = take(c.cap * 4);
+  c.eids = take((c.cap + kDenseBlock - 1) / kDenseBlock * 4);
+  c.npp = take(4);
+  if (inter > 0) {
+    c.act = take(m * inter * 2);
+    c.act_q = take(m * inter);
+    c.a2 = take(m * 4);
+  }
+  c.total = off;
+  return c;
+}
+
+int dense_prologue(const void* x, int64_t m, int k, void* workspace, int64_t workspace_bytes,
+                   const DenseCarve& c, void* stream) {
+  if (m > INT32_MAX - kDenseBlock) return fail(MOE_I8_EINVAL, "too many rows");
+  if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(MOE_I8_EINVAL, "workspace must be 256-byte aligned");
+  if (workspace_bytes < c.total)
+    return fail(MOE_I8_EWORKSPACE, "workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)c.total);
+  char* ws = static_cast<char*>(workspace);
+  if (int rc = moe_i8_scaled_int8_quant(x, MOE_I8_DTYPE_BF16, m, k, k, reinterpret_cast<int8_t*>(ws + c.x_q),
+                                        reinterpret_cast<float*>(ws + c.a1), stream))
+    return rc;
+  return check_launch(
+      moe_i8::launch_identity_routing((int)m, kDenseBlock, c.cap, reinterpret_cast<int32_t*>(ws + c.sorted),
+                                      reinterpret_cast<int32_t*>(ws + c.eids),
+                                      reinterpret_cast<int32_t*>(ws + c.npp), static_cast<hipStream_t>(stream)),
+      "identity_routing");
+}
+}  // namespace
+
+int64_t moe_i8_dense_workspace_bytes(int64_t m, int k, int inter) {
+  if (m < 0 || k < 1 || inter < 0) return -1;
+  return dense_carve(m, k, inter).total;
+}
+
+int moe_i8_w8a8_linear(const void* x, const int8_t* w, const float* w_scale, void* out, int64_t m, int n,
+                       int k, void* workspace, int64_t workspace_bytes, int variant, void* stream) {
+  if (m < 0) return fail(MOE_I8_EINVAL, "negative m");
+  if (m == 0) return MOE_I8_OK;
+  if (!x || !w || !w_scale || !out || !workspace) return fail(MOE_I8_EINVAL, "null pointer");
+  const DenseCarve c = dense_carve(m, k, 0);
+  if (int rc = dense_prologue(x, m, k, workspace, workspace_bytes, c, stream)) return rc;
+  char* ws = static_cast<char*>(workspace);
+  return moe_i8_gemm_down(reinterpret_cast<int8_t*>(ws + c.x_q), reinterpret_cast<float*>(ws + c.a1), w, w_scale,
+                          nullptr, reinterpret_cast<int32_t*>(ws + c.sorted), reinterpret_cast<int32_t*>(ws + c.eids),
+                          reinterpret_cast<int32_t*>(ws + c.npp), m, 1, n, k, kDenseBlock, c.cap, out, variant,
+                          stream);
+}
+
+int moe_i8_w8a8_mlp(const void* x, const int8_t* w13, const float* w13_scale, const int8_t* w2,
+                    const float* w2_scale, void* out, int64_t m, int hidden, int inter, void* workspace,
+                    int64_t workspace_bytes, int variant, void* stream) {
+  if (m < 0) return fail(MOE_I8_EINVAL, "negative m");
+  if (m == 0) return MOE_I8_OK;
+  if (!x || !w13 || !w13_scale || !w2 || !w2_scale || !out || !workspace) return fail(MOE_I8_EINVAL, "null pointer");
+  if (inter < 64 || inter % 64) return fail(MOE_I8_EINVAL, "inter (%d) must be a positive multiple of 64", inter);
+  const DenseCarve c = dense_carve(m, hidden, inter);
+  if (int rc = dense_prologue(x, m, hidden, workspace, workspace_bytes, c, stream)) return rc;
+  char* ws = static_cast<char*>(workspace);
+  int8_t* x_q = reinterpret_cast<int8_t*>(ws + c.x_q);
+  float* a1 = reinterpret_cast<float*>(ws + c.a1);
+  int32_t* sorted = reinterpret_cast<int32_t*>(ws + c.sorted);
+  int32_t* eids = reinterpret_cast<int32_t*>(ws + c.eids);
+  int32_t* npp = reinterpret_cast<int32_t*>(ws + c.npp);
+  int8_t* act_q = reinterpret_cast<int8_t*>(ws + c.act_q);
+  float* a2 = reinterpret_cast<float*>(ws + c.a2);
+  if (int rc = moe_i8_gemm_gate_up_silu(x_q, a1, w13, w13_scale, sorted, eids, npp, m, 1, 1, hidden, inter,
+                                        kDenseBlock, c.cap, ws + c.act, variant, stream))
+    return rc;
+  if (int rc = moe_i8_scaled_int8_quant(ws + c.act, MOE_I8_DTYPE_BF16, m, inter, inter, act_q, a2, stream)) return rc;
+  return moe_i8_gemm_down(act_q, a2, w2, w2_scale, nullptr, sorted, eids, npp, m, 1, hidden, inter, kDenseBlock,
+                          c.cap, out, variant, stream);
 }
 
 }  // extern "C"

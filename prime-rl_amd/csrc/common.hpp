@@ -131,6 +131,7 @@ struct QuantArgs {
   int64_t rows_per_group = 0;
   int64_t out_rows_per_group = 0;
   int64_t out_row_offset = 0;
+  int round_even = 0;  // activations: ties to even instead of away from zero
 };
 hipError_t launch_quant_rows(const QuantArgs& a, hipStream_t stream);
 // Router: scores -> (grouped) top-k -> weights, one wavefront per token.
@@ -160,6 +161,8 @@ hipError_t launch_route_topk(const RouteArgs& a, hipStream_t stream);
 // Per-output-channel weight quantisation (round to nearest even of w / scale, scale = absmax / 127).
 hipError_t launch_quant_weights(const QuantArgs& a, hipStream_t stream);
 // moe_align and the quantisation of `q` in one launch; only when align_quant_fusable() says so.
+hipError_t launch_identity_routing(int rows, int block_size, int64_t sorted_cap, int32_t* sorted,
+                                   int32_t* expert_ids, int32_t* npp, hipStream_t stream);
 bool align_quant_fusable(const AlignArgs& a, const QuantArgs& q);
 hipError_t launch_align_quant(const AlignArgs& a, const QuantArgs& q, hipStream_t stream);
 
@@ -171,7 +174,7 @@ struct GemmArgs {
   const float* a_scale;   // per activation row
   const int8_t* w;        // [E, N, K]
   const float* w_scale;   // [E, N]
-  const float* row_weight;  // [P] routed weights (down) or null
+  const float* row_weight;  // [P] routed weights (down); null = 1
   const int32_t* sorted_token_ids;
   const int32_t* expert_ids;
   const int32_t* num_tokens_post_padded;

@@ -158,7 +158,7 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
       for (int s = 0; s < NS; ++s) {
         if (!tok_ok[s]) continue;
         const float as = p.a_scale[tok[s] / p.row_div];
-        const float rw = p.row_weight[tok[s]];
+        const float rw = p.row_weight ? p.row_weight[tok[s]] : 1.0f;
 #pragma unroll
         for (int t = 0; t < kTiles; ++t) {
           if (!wok[t]) continue;

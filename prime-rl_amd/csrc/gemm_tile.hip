@@ -287,7 +287,7 @@ __device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, in
     for (int tj = 0; tj < 2; ++tj) {
       // 32 token rows x 128 channels: rows of 256 bytes = 16 chunks
       const float as = tok[tj] >= 0 ? p.a_scale[tok[tj] / p.row_div] : 0.0f;
-      const float rw = tok[tj] >= 0 ? p.row_weight[tok[tj]] : 0.0f;
+      const float rw = tok[tj] >= 0 ? (p.row_weight ? p.row_weight[tok[tj]] : 1.0f) : 0.0f;
 #pragma unroll
       for (int ci = 0; ci < 4; ++ci) {
 #pragma unroll

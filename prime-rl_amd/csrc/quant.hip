@@ -15,10 +15,22 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kRowsPerBlock = kThreads / kWave;
 
-template <int VPL>
+template <int VPL, int kMode>
 __global__ __launch_bounds__(kThreads) void quant_rows_kernel(QuantArgs a) {
   const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
-  if (row < a.rows) quant_one_row<VPL>(a, row);
+  if (row < a.rows) quant_one_row<VPL, kMode>(a, row);
+}
+
+template <int kMode>
+void launch_quant_rows_mode(const QuantArgs& a, dim3 grid, dim3 block, hipStream_t stream) {
+  switch (quant_vectors_per_lane(a.cols)) {
+    case 1: hipLaunchKernelGGL((quant_rows_kernel<1, kMode>), grid, block, 0, stream, a); break;
+    case 2: hipLaunchKernelGGL((quant_rows_kernel<2, kMode>), grid, block, 0, stream, a); break;
+    case 4: hipLaunchKernelGGL((quant_rows_kernel<4, kMode>), grid, block, 0, stream, a); break;
+    case 8: hipLaunchKernelGGL((quant_rows_kernel<8, kMode>), grid, block, 0, stream, a); break;
+    case 16: hipLaunchKernelGGL((quant_rows_kernel<16, kMode>), grid, block, 0, stream, a); break;
+    default: hipLaunchKernelGGL((quant_rows_kernel<0, kMode>), grid, block, 0, stream, a); break;
+  }
 }
 
 // Weights: rows are contiguous and there are many of them, so a wavefront walks kWeightRowsPerWave
@@ -110,7 +122,7 @@ __global__ __launch_bounds__(kThreads) void quant_weights_kernel(QuantArgs a) {
 // Rows too long to hold in registers: one wavefront per row, read twice.
 __global__ __launch_bounds__(kThreads) void quant_weights_long_rows_kernel(QuantArgs a) {
   const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
-  if (row < a.rows) quant_one_row<0, true>(a, row);
+  if (row < a.rows) quant_one_row<0, kQuantWeights>(a, row);
 }
 
 }  // namespace
@@ -119,14 +131,10 @@ hipError_t launch_quant_rows(const QuantArgs& a, hipStream_t stream) {
   if (a.rows == 0) return hipSuccess;
   const dim3 grid((unsigned)((a.rows + kRowsPerBlock - 1) / kRowsPerBlock));
   const dim3 block(kThreads);
-  switch (quant_vectors_per_lane(a.cols)) {
-    case 1: hipLaunchKernelGGL(quant_rows_kernel<1>, grid, block, 0, stream, a); break;
-    case 2: hipLaunchKernelGGL(quant_rows_kernel<2>, grid, block, 0, stream, a); break;
-    case 4: hipLaunchKernelGGL(quant_rows_kernel<4>, grid, block, 0, stream, a); break;
-    case 8: hipLaunchKernelGGL(quant_rows_kernel<8>, grid, block, 0, stream, a); break;
-    case 16: hipLaunchKernelGGL(quant_rows_kernel<16>, grid, block, 0, stream, a); break;
-    default: hipLaunchKernelGGL(quant_rows_kernel<0>, grid, block, 0, stream, a); break;
-  }
+  if (a.round_even)
+    launch_quant_rows_mode<kQuantEven>(a, grid, block, stream);
+  else
+    launch_quant_rows_mode<kQuantAway>(a, grid, block, stream);
   return hipGetLastError();
 }
 

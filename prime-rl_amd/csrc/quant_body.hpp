@@ -21,13 +21,16 @@ __device__ __forceinline__ float absmax8(const uint4& v) {
   return m;
 }
 
+// kEven: ties to even (rintf) instead of away from zero (roundf).
+template <bool kEven = false>
 __device__ __forceinline__ uint2 quant8(const uint4& v, float inv) {
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
   uint32_t out[2] = {0u, 0u};
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int lo = (int)roundf(__uint_as_float(w[i] << 16) * inv);
-    const int hi = (int)roundf(__uint_as_float(w[i] & 0xffff0000u) * inv);
+    const float flo = __uint_as_float(w[i] << 16) * inv, fhi = __uint_as_float(w[i] & 0xffff0000u) * inv;
+    const int lo = (int)(kEven ? rintf(flo) : roundf(flo));
+    const int hi = (int)(kEven ? rintf(fhi) : roundf(fhi));
     const uint32_t pair = ((uint32_t)lo & 0xffu) | (((uint32_t)hi & 0xffu) << 8);
     out[i >> 1] |= pair << ((i & 1) * 16);
   }
@@ -98,9 +101,11 @@ __device__ __forceinline__ uint2 quant8_weights(const uint4& v, const WeightRcp&
 
 // VPL = 16-byte vectors per lane held in registers (covers cols <= VPL * 512).
 // VPL == 0: rows of any length, read twice (second read served by the caches).
-// kWeights: per-output-channel weight quantisation instead of the activation arithmetic:
-// scale = max(absmax / 127, 1e-12), q = clamp(rint(x / scale), +-127).
-template <int VPL, bool kWeights = false>
+// kMode: kQuantAway = activations, q = roundf(x * (127 / absmax)) (ties away from zero);
+// kQuantEven = the same with ties to even; kQuantWeights = per-output-channel weights,
+// scale = max(absmax / 127, 1e-12), q = rint(x / scale).
+enum QuantMode { kQuantAway = 0, kQuantWeights = 1, kQuantEven = 2 };
+template <int VPL, int kMode = kQuantAway>
 __device__ __forceinline__ void quant_one_row(const QuantArgs& a, int64_t row) {
   const int lane = lane_id();
   const int64_t src = a.gather ? (int64_t)(a.gather[row] / a.gather_div) : row;
@@ -122,7 +127,7 @@ __device__ __forceinline__ void quant_one_row(const QuantArgs& a, int64_t row) {
     float m = 0.0f;
 #pragma unroll
     for (int i = 0; i < VPL; ++i) m = fmaxf(m, absmax8(v[i]));
-    if constexpr (kWeights) {
+    if constexpr (kMode == kQuantWeights) {
       const WeightRcp s = weight_rcp(fmaxf(wave_max(m) / 127.0f, 1e-12f));
       if (lane == 0) a.scale[orow] = s.scale;
 #pragma unroll
@@ -137,14 +142,14 @@ __device__ __forceinline__ void quant_one_row(const QuantArgs& a, int64_t row) {
 #pragma unroll
       for (int i = 0; i < VPL; ++i) {
         const int c = lane + i * kWave;
-        if (c < nvec) out[c] = quant8(v[i], inv);
+        if (c < nvec) out[c] = quant8<kMode == kQuantEven>(v[i], inv);
       }
     }
   } else {
     float m = 0.0f;
     if (have)
       for (int c = lane; c < nvec; c += kWave) m = fmaxf(m, absmax8(in[c]));
-    if constexpr (kWeights) {
+    if constexpr (kMode == kQuantWeights) {
       const WeightRcp s = weight_rcp(fmaxf(wave_max(m) / 127.0f, 1e-12f));
       if (lane == 0) a.scale[orow] = s.scale;
       for (int c = lane; c < nvec; c += kWave) out[c] = have ? quant8_weights(in[c], s) : make_uint2(0u, 0u);
@@ -153,7 +158,7 @@ __device__ __forceinline__ void quant_one_row(const QuantArgs& a, int64_t row) {
       const float inv = 127.0f / absmax;
       if (lane == 0) a.scale[orow] = absmax / 127.0f;
       for (int c = lane; c < nvec; c += kWave)
-        out[c] = have ? quant8(in[c], inv) : make_uint2(0u, 0u);
+        out[c] = have ? quant8<kMode == kQuantEven>(in[c], inv) : make_uint2(0u, 0u);
     }
   }
 }
