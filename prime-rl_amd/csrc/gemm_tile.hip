@@ -255,7 +255,7 @@ __device__ __forceinline__ void multiply_stage(const TileReads& rd, const char* 
 // so that neither the 8-byte writes nor the 16-byte reads pile up on a bank).
 template <int MODE>
 __device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, int chh, int tb, int lane,
-                                         v16i (&acc)[4][2], char* wave_lds) {
+                                         v16i (&acc)[4][2], char* wave_lds, float* wave_scales) {
   const int lrow = lane & 31;
   const int lhalf = lane >> 5;
   const int inter = p.N / 2;
@@ -283,23 +283,37 @@ __device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, in
   } else if constexpr (MODE == kDown) {
     const float* wsc = p.w_scale + (int64_t)tk.e * p.N;
     const int n0 = tk.nt * kBN + chh * 128;  // first channel of this wavefront
+    // The 128 channel scales of this wavefront go through LDS: read from there they do not count
+    // as vector-memory loads, so the second half's arithmetic does not have to wait for the first
+    // half's stores (the vector-memory counter retires in order).
+    {
+      const int n = n0 + 2 * lane;
+      *reinterpret_cast<float2*>(wave_scales + 2 * lane) =
+          n < p.N ? *reinterpret_cast<const float2*>(wsc + n) : make_float2(0.0f, 0.0f);
+    }
+    float as[2], rw[2];
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+      as[tj] = tok[tj] >= 0 ? p.a_scale[tok[tj] / p.row_div] : 0.0f;
+      rw[tj] = tok[tj] >= 0 ? (p.row_weight ? p.row_weight[tok[tj]] : 1.0f) : 0.0f;
+    }
 #pragma unroll
     for (int tj = 0; tj < 2; ++tj) {
       // 32 token rows x 128 channels: rows of 256 bytes = 16 chunks
-      const float as = tok[tj] >= 0 ? p.a_scale[tok[tj] / p.row_div] : 0.0f;
-      const float rw = tok[tj] >= 0 ? (p.row_weight ? p.row_weight[tok[tj]] : 1.0f) : 0.0f;
 #pragma unroll
       for (int ci = 0; ci < 4; ++ci) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int n = n0 + ci * 32 + 8 * q + 4 * lhalf;
-          const float4 ws = *reinterpret_cast<const float4*>(wsc + (n < p.N ? n : 0));
+          const float4 ws = *reinterpret_cast<const float4*>(wave_scales + ci * 32 + 8 * q + 4 * lhalf);
           const int v[4] = {acc[ci][tj][4 * q], acc[ci][tj][4 * q + 1], acc[ci][tj][4 * q + 2], acc[ci][tj][4 * q + 3]};
           *reinterpret_cast<uint2*>(wave_lds + lrow * 256 + (((ci * 4 + q) ^ (lrow & 15)) * 16) + lhalf * 8) =
-              down_epilogue4(v, as, ws, rw);
+              down_epilogue4(v, as[tj], ws, rw[tj]);
         }
-        __builtin_amdgcn_sched_barrier(0);  // keep the scale loads of later groups from piling up in VGPRs
       }
+      // Before the first stores everything this wavefront has in flight is complete (its share of
+      // the next tile's first stage, issued during the last step, and the loads above), so the
+      // stores are the only vector-memory work still pending when the next tile starts.
+      if (tj == 0) wait_vmcnt<0>();
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
         const int row = r * 4 + (lane >> 4);
@@ -334,6 +348,7 @@ __device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, in
               silu_mul_epilogue4(g, u, as, wg, wu);
         }
     }
+    wait_vmcnt<0>();  // as in the down epilogue: only the stores below stay pending
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
       const int row = r * 8 + (lane >> 3);
@@ -352,6 +367,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(TileParams p) {
   __shared__ __align__(16) char stages[2 * kStageBytes];
   __shared__ uint32_t tile_desc[kMaxTiles];
   __shared__ int wave_part[kWaves];
+  __shared__ __align__(16) float channel_scales[kWaves * 128];
   __shared__ int total_tiles;
 
   const int t = threadIdx.x;
@@ -423,6 +439,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(TileParams p) {
   // with a barrier), so the first stage can be filled now.
   issue_stage_loads(ld, p.a_q, stage0, wave, 0, my_tokens);
 
+  bool stores_pending = false;
   while (true) {
     v16i acc[4][2];
 #pragma unroll
@@ -441,8 +458,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(TileParams p) {
     const bool nx_tokens = tb < nx.nsub;
 
     for (int s = 0; s < nk; ++s) {
-      // this wavefront's loads of step s have landed (nothing newer is in flight) ...
-      wait_vmcnt<0>();
+      // this wavefront's loads of step s have landed (nothing newer is in flight) ...  A wavefront
+      // that has just run an epilogue waited for its loads there and only has the epilogue's
+      // stores pending: it lets them drain behind the first step instead of stalling on them.
+      if (s > 0 || !stores_pending) wait_vmcnt<0>();
       // ... and so have everybody's; everybody is also done reading the other stage
       __builtin_amdgcn_s_barrier();
       const uint32_t other = stage0 + (parity ^ 1) * kStageBytes;
@@ -456,7 +475,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(TileParams p) {
     // everybody is done reading the stage of the last step: it becomes the epilogue's staging area
     // (the next task's first loads went to the other stage)
     __builtin_amdgcn_s_barrier();
-    if (my_tokens) epilogue<MODE>(p, tk, chh, tb, lane, acc, stages + (parity ^ 1) * kStageBytes + wave * 8192);
+    if (my_tokens)
+      epilogue<MODE>(p, tk, chh, tb, lane, acc, stages + (parity ^ 1) * kStageBytes + wave * 8192,
+                     channel_scales + wave * 128);
+    stores_pending = my_tokens && MODE != kAccI32;
     if (nx.e < 0) break;
     tk = nx;
     ld = nld;
