@@ -241,7 +241,7 @@ __global__ __launch_bounds__(kMultiThreads) void align_hist_kernel(
   }
 }
 
-__global__ __launch_bounds__(kSingleThreads) void align_scan_kernel(
+__device__ __forceinline__ void align_scan_body(
     int E, int B, int units, const int32_t* __restrict__ unit_hist, int32_t* __restrict__ unit_base,
     int32_t* __restrict__ seg_out, int32_t* __restrict__ expert_ids, int64_t expert_cap,
     int32_t* __restrict__ npp_out) {
@@ -272,6 +272,28 @@ __global__ __launch_bounds__(kSingleThreads) void align_scan_kernel(
   }
   __syncthreads();
   write_expert_ids(seg, E, B, npp, expert_ids, expert_cap);
+}
+
+__global__ __launch_bounds__(kSingleThreads) void align_scan_kernel(
+    int E, int B, int units, const int32_t* __restrict__ unit_hist, int32_t* __restrict__ unit_base,
+    int32_t* __restrict__ seg_out, int32_t* __restrict__ expert_ids, int64_t expert_cap,
+    int32_t* __restrict__ npp_out) {
+  align_scan_body(E, B, units, unit_hist, unit_base, seg_out, expert_ids, expert_cap, npp_out);
+}
+
+// The scan is one workgroup; the quantisation of the layer input, which does not depend on the
+// routing, fills the rest of the machine in the same launch (workgroups >= 1, 16 rows each).
+template <int VPL>
+__global__ __launch_bounds__(kSingleThreads) void align_scan_quant_kernel(
+    int E, int B, int units, const int32_t* __restrict__ unit_hist, int32_t* __restrict__ unit_base,
+    int32_t* __restrict__ seg_out, int32_t* __restrict__ expert_ids, int64_t expert_cap,
+    int32_t* __restrict__ npp_out, QuantArgs q) {
+  if (blockIdx.x == 0) {
+    align_scan_body(E, B, units, unit_hist, unit_base, seg_out, expert_ids, expert_cap, npp_out);
+    return;
+  }
+  const int64_t row = (int64_t)(blockIdx.x - 1) * kSingleWaves + threadIdx.x / kWave;
+  if (row < q.rows) quant_one_row<VPL>(q, row);
 }
 
 __global__ __launch_bounds__(kMultiThreads) void align_scatter_kernel(
@@ -313,7 +335,8 @@ int64_t align_workspace_ints(int64_t num_pairs, int num_experts) {
 }
 
 bool align_quant_fusable(const AlignArgs& a, const QuantArgs& q) {
-  return a.num_pairs <= kSingleMaxPairs && q.rows > 0 && q.rows <= kSingleMaxPairs;
+  if (q.rows <= 0 || q.rows > (int64_t)kSingleWaves * 0x7ffffff0) return false;
+  return a.num_pairs > kSingleMaxPairs || q.rows <= kSingleMaxPairs;
 }
 
 namespace {
@@ -324,6 +347,37 @@ constexpr int kSingleLdsMax = (int)(sizeof(int) * ((size_t)kSingleWaves * kMaxEx
 hipError_t launch_align_quant(const AlignArgs& a, const QuantArgs& q, hipStream_t stream) {
   const int E = a.num_experts;
   const dim3 grid(1 + (unsigned)((q.rows + kSingleWaves - 1) / kSingleWaves));
+  if (a.num_pairs > kSingleMaxPairs) {
+    // three launches as launch_align, the middle one (a single scanning workgroup) also quantises
+    const int nbits = bits_for(E);
+    const int units = (int)((a.num_pairs + kMultiChunk - 1) / kMultiChunk);
+    int32_t* unit_hist = a.workspace;
+    int32_t* unit_base = unit_hist + (int64_t)units * E;
+    int32_t* seg = unit_base + (int64_t)units * E;
+    const size_t lds = sizeof(int) * (size_t)kMultiWaves * E;
+    hipLaunchKernelGGL(align_hist_kernel, dim3(units), dim3(kMultiThreads), lds, stream, a.topk_ids,
+                       a.num_pairs, E, nbits, unit_hist, a.sorted_token_ids, a.sorted_cap);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return err;
+#define MOE_I8_SCAN_QUANT(V)                                                                           \
+  hipLaunchKernelGGL(align_scan_quant_kernel<V>, grid, dim3(kSingleThreads), 0, stream, E, a.block_size, \
+                     units, unit_hist, unit_base, seg, a.expert_ids, a.expert_cap, a.num_tokens_post_padded, q)
+    switch (quant_vectors_per_lane(q.cols)) {
+      case 1: MOE_I8_SCAN_QUANT(1); break;
+      case 2: MOE_I8_SCAN_QUANT(2); break;
+      case 4: MOE_I8_SCAN_QUANT(4); break;
+      case 8: MOE_I8_SCAN_QUANT(8); break;
+      case 16: MOE_I8_SCAN_QUANT(16); break;
+      default: MOE_I8_SCAN_QUANT(0); break;
+    }
+#undef MOE_I8_SCAN_QUANT
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    hipLaunchKernelGGL(align_scatter_kernel, dim3(units), dim3(kMultiThreads), lds, stream,
+                       a.topk_ids, a.num_pairs, E, nbits, unit_base, seg, a.sorted_token_ids,
+                       a.sorted_cap);
+    return hipGetLastError();
+  }
 #define MOE_I8_FUSED_LAUNCH(V)                                                                      \
   do {                                                                                              \
     static const hipError_t attr = hipFuncSetAttribute((const void*)align_quant_kernel<V>,          \

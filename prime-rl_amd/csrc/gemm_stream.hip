@@ -81,13 +81,53 @@ __device__ __forceinline__ void pair_rows(const StreamParams& p, int q, int (&wr
   }
 }
 
+// `count_valid`: first pass over a block; the number of valid rows of the block is counted here,
+// after the first weight window has been requested, and returned.
 template <int MODE, int NS>
-__device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int e, int sub0, int first_pair,
-                                            int npairs, char* wave_lds) {
+__device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e, int sub0, int first_pair,
+                                           int npairs, char* wave_lds, bool count_valid) {
   const int lane = lane_id();
   const int col = lane & 15;  // token slot inside a sub-tile / weight row inside a tile
   const int grp = lane >> 4;  // which 16 reduction bytes of each step; which 4 output channels
   const int K = p.K;
+
+  // Load j of a window covers rows 4 * (j % 4) + (lane >> 4) of tile j / 4, chunk lane & 15.
+  const int ld_row = lane >> 4;
+  const int ld_chunk = lane & 15;
+  const int8_t* wbase = p.w + ((int64_t)e * p.N + ld_row) * K + ld_chunk * 16;
+  // LDS: [32 rows][256 B]; chunk c of row r sits at position c ^ (r & 15)
+  const int st_base = ld_row * kWinBytes + ((ld_chunk ^ ld_row) * 16);  // ^ (j % 4) * 64, + j * 1024
+  const int rd_base = col * kWinBytes + ((grp ^ col) * 16);             // ^ u * 64, + t * 4096
+
+  // The wavefront walks windows (pair 0, k 0), (pair 0, k 256), ..., (pair 1, k 0), ... ; `fq`/`fk`
+  // track the window being fetched, `cq`/`ck` the one being consumed.
+  int fq = 0, fk = 0;
+  auto fetch_weights = [&](Window<NS>& win) {
+    int wrow[kTiles];
+    bool wok[kTiles];
+    pair_rows<MODE>(p, first_pair + fq, wrow, wok);
+    const bool chunk_in = fk + ld_chunk * 16 < K;  // only the last window of a ragged K is partial
+#pragma unroll
+    for (int j = 0; j < kWinLoads; ++j) {
+      const int8_t* src = wbase + (int64_t)(wrow[j / 4] + 4 * (j % 4)) * K + fk;
+      win.w[j] = chunk_in ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src)) : v4i{0, 0, 0, 0};
+    }
+  };
+
+  // The weights of the first window depend on nothing but the expert of the block: they are
+  // requested from HBM before the chain of dependent reads (row list -> token -> activation row)
+  // that the rest of the set-up is.
+  Window<NS> w0, w1;
+  fetch_weights(w0);
+
+  int nvalid = 0;
+  if (count_valid) {
+    for (int base = 0; base < p.B; base += kWave) {
+      const int slot = base + lane;
+      const int32_t t = slot < p.B ? p.sorted_ids[(int64_t)blk * p.B + slot] : -1;
+      nvalid += __popcll(__ballot(t >= 0 && t < p.P));
+    }
+  }
 
   int32_t tok[NS];
   bool tok_ok[NS];
@@ -99,13 +139,6 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
     const int64_t arow = tok_ok[s] ? tok[s] / p.row_div : 0;
     ap[s] = p.a_q + arow * K + grp * 16;
   }
-  // Load j of a window covers rows 4 * (j % 4) + (lane >> 4) of tile j / 4, chunk lane & 15.
-  const int ld_row = lane >> 4;
-  const int ld_chunk = lane & 15;
-  const int8_t* wbase = p.w + ((int64_t)e * p.N + ld_row) * K + ld_chunk * 16;
-  // LDS: [32 rows][256 B]; chunk c of row r sits at position c ^ (r & 15)
-  const int st_base = ld_row * kWinBytes + ((ld_chunk ^ ld_row) * 16);  // ^ (j % 4) * 64, + j * 1024
-  const int rd_base = col * kWinBytes + ((grp ^ col) * 16);             // ^ u * 64, + t * 4096
 
   v4i acc[kTiles][NS];
 #pragma unroll
@@ -113,19 +146,7 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
 #pragma unroll
     for (int s = 0; s < NS; ++s) acc[t][s] = v4i{0, 0, 0, 0};
 
-  // The wavefront walks windows (pair 0, k 0), (pair 0, k 256), ..., (pair 1, k 0), ... ; `fq`/`fk`
-  // track the window being fetched, `cq`/`ck` the one being consumed.
-  int fq = 0, fk = 0;
-  auto fetch = [&](Window<NS>& win) {
-    int wrow[kTiles];
-    bool wok[kTiles];
-    pair_rows<MODE>(p, first_pair + fq, wrow, wok);
-    const bool chunk_in = fk + ld_chunk * 16 < K;  // only the last window of a ragged K is partial
-#pragma unroll
-    for (int j = 0; j < kWinLoads; ++j) {
-      const int8_t* src = wbase + (int64_t)(wrow[j / 4] + 4 * (j % 4)) * K + fk;
-      win.w[j] = chunk_in ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src)) : v4i{0, 0, 0, 0};
-    }
+  auto fetch_rows = [&](Window<NS>& win) {
 #pragma unroll
     for (int s = 0; s < NS; ++s)
 #pragma unroll
@@ -137,6 +158,10 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
       fk = 0;
       ++fq;
     }
+  };
+  auto fetch = [&](Window<NS>& win) {
+    fetch_weights(win);
+    fetch_rows(win);
   };
 
   // Epilogue of one tile pair: lane holds channels wrow[t] + 4 * grp + {0..3} of token tok[s].
@@ -216,8 +241,7 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
 
   const int nwin = (K + kWinBytes - 1) / kWinBytes;
   const int total = npairs * nwin;
-  Window<NS> w0, w1;
-  fetch(w0);
+  fetch_rows(w0);
   for (int i = 0; i < total; i += 2) {
     if (i + 1 < total) fetch(w1);
     consume(w0);
@@ -225,6 +249,7 @@ __device__ __forceinline__ void stream_pass(const StreamParams& p, int blk, int 
     if (i + 2 < total) fetch(w0);
     consume(w1);
   }
+  return nvalid;
 }
 
 // grid.x: groups of kWaves wavefronts along the weight rows; grid.y: 64-row (B-row) blocks.
@@ -242,17 +267,13 @@ __global__ __launch_bounds__(kThreads, 3) void gemm_stream_kernel(StreamParams p
   if (first_pair >= total_pairs) return;
   const int npairs = total_pairs - first_pair < p.pairs_per_wave ? total_pairs - first_pair : p.pairs_per_wave;
 
-  // Valid rows are a prefix of the block: count them to know how many sub-tiles to run.
-  int nvalid = 0;
-  for (int base = 0; base < p.B; base += kWave) {
-    const int slot = base + lane;
-    const int32_t t = slot < p.B ? p.sorted_ids[(int64_t)blk * p.B + slot] : -1;
-    nvalid += __popcll(__ballot(t >= 0 && t < p.P));
-  }
-  const int nsub = (nvalid + kSub - 1) / kSub;
+  // Valid rows are a prefix of the block (at least one, the block is in use): the first pass counts
+  // them to know how many sub-tiles there are.
   char* wave_lds = lds + (threadIdx.x / kWave) * kWaveLds;
-  for (int sub0 = 0; sub0 < nsub; sub0 += kGroup)
-    stream_pass<MODE, kGroup>(p, blk, e, sub0, first_pair, npairs, wave_lds);
+  const int nvalid = stream_pass<MODE, kGroup>(p, blk, e, 0, first_pair, npairs, wave_lds, true);
+  const int nsub = (nvalid + kSub - 1) / kSub;
+  for (int sub0 = kGroup; sub0 < nsub; sub0 += kGroup)
+    stream_pass<MODE, kGroup>(p, blk, e, sub0, first_pair, npairs, wave_lds, false);
 }
 
 template <int MODE>

@@ -35,6 +35,7 @@ constexpr int kTokOffset = kBN * kBK;
 constexpr int kStageBytes = (kBN + kTileTok) * kBK;  // 64 KB
 constexpr int kMaxTiles = 6144;                      // capacity of the in-LDS tile list
 constexpr int kXcds = 8;
+constexpr int kGroupTiles = 8;  // token tiles of one expert whose tasks are interleaved per channel tile
 
 struct TileParams {
   const int8_t* a_q;
@@ -112,8 +113,9 @@ __device__ __forceinline__ void block_scan(int v, int* wave_part, int& incl, int
   excl = scan_op<kMax>(carry, prev);
 }
 
-// tile_desc[t] = first block | number of blocks << 16.  Tiles start at multiples of `per_tile`
-// blocks inside each run of equal expert ids and never cross a run.  scratch holds nblocks ints.
+// tile_desc[t] = first block | number of blocks << 16 | rank in group << 20 | group size << 24.
+// Tiles start at multiples of `per_tile` blocks inside each run of equal expert ids and never cross
+// a run; up to kGroupTiles consecutive tiles of a run form a group.  scratch holds nblocks ints.
 __device__ int build_tile_list(const int32_t* __restrict__ expert_ids, int nblocks, int per_tile, int* scratch,
                                int* wave_part, uint32_t* tile_desc, int* total_out) {
   const int tid = threadIdx.x;
@@ -142,13 +144,25 @@ __device__ int build_tile_list(const int32_t* __restrict__ expert_ids, int nbloc
     if ((j - cur) % per_tile == 0) {
       int nb = 1;
       while (nb < per_tile && j + nb < nblocks && scratch[j + nb] == scratch[j]) ++nb;
-      if (t < kMaxTiles) tile_desc[t] = (uint32_t)j | ((uint32_t)nb << 16);
+      // bits 0-15 first block, 16-19 blocks, 20-22 rank of the tile inside its group, 24-27 group size
+      if (t < kMaxTiles)
+        tile_desc[t] = (uint32_t)j | ((uint32_t)nb << 16) | ((uint32_t)(((j - cur) / per_tile) % kGroupTiles) << 20);
       ++t;
     }
   }
   if (tid == kThreads - 1) *total_out = incl_leaders < kMaxTiles ? incl_leaders : kMaxTiles;
   __syncthreads();
-  return *total_out;
+  // Groups: up to kGroupTiles consecutive tiles of one expert.  The leader of a group counts its
+  // members and writes the size into all of them.
+  const int total = *total_out;
+  for (int g = tid; g < total; g += kThreads) {
+    if (((tile_desc[g] >> 20) & 7u) != 0) continue;
+    int count = 1;
+    while (count < kGroupTiles && g + count < total && ((tile_desc[g + count] >> 20) & 7u) == (uint32_t)count) ++count;
+    for (int i = 0; i < count; ++i) tile_desc[g + i] |= (uint32_t)count << 24;
+  }
+  __syncthreads();
+  return total;
 }
 
 struct Task {
@@ -416,12 +430,19 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(TileParams p) {
     tk.nsub = 0;
     if (it < per_xcd && xcd * per_xcd + it < total) {
       const int task = xcd * per_xcd + it;
-      const uint32_t d = tile_desc[task / p.ntiles];
+      // The tasks of a group of T token tiles of one expert run channel tile by channel tile: T
+      // consecutive tasks (on neighbouring compute units) stream the same weight tile.
+      const int tile0 = task / p.ntiles;
+      const uint32_t d0 = tile_desc[tile0];
+      const int first = tile0 - (int)((d0 >> 20) & 7u);
+      const int T = (int)((d0 >> 24) & 15u);
+      const int pos = task - first * p.ntiles;
+      const uint32_t d = tile_desc[first + pos % T];
+      tk.nt = pos / T;
       const int blk = (int)(d & 0xffffu);
       const int e = p.expert_ids[blk];
-      tk.nt = task % p.ntiles;
       tk.slot0 = (int64_t)blk * p.B;
-      tk.nsub = (int)(d >> 16) * sub_per_block;
+      tk.nsub = (int)((d >> 16) & 15u) * sub_per_block;
       tk.e = (e >= 0 && e < p.E) ? e : -2;
     }
     return tk;
