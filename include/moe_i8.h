@@ -151,6 +151,17 @@ int moe_i8_gemm_down(const int8_t* h_q, const float* a_scale, const int8_t* w2,
                      int variant, void* stream);
 
 /*
+ * The down GEMM with the second `per_token_quant_int8` folded in (streaming family only, inter <= 1024):
+ * act bf16 [num_pairs, I] is quantised row by row inside the kernel with the arithmetic of
+ * moe_i8_quant_rows, so the result equals moe_i8_quant_rows followed by moe_i8_gemm_down bit for bit.
+ * moe_i8_fused_experts uses it whenever it picks the streaming family for the down GEMM.
+ */
+int moe_i8_gemm_down_bf16(const void* act, const int8_t* w2, const float* w2_scale, const float* topk_weights,
+                          const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                          const int32_t* num_tokens_post_padded, int64_t num_pairs, int num_experts, int hidden,
+                          int inter, int block_size, int64_t sorted_cap, void* out, void* stream);
+
+/*
  * Raw int32 accumulators of either grouped GEMM (inspection / parity only):
  * acc[t, n] = sum_K a_q[t / row_div, K] * w[e_t, n, K] for every routed pair t.
  * a_q int8 [*, K], w int8 [E, N, K] -> acc int32 [num_pairs, N].

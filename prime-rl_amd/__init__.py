@@ -17,6 +17,7 @@ from .api import (  # noqa: F401
     w8a8_mlp,
     gemm_acc_i32,
     gemm_down,
+    gemm_down_bf16,
     gemm_gate_up_silu,
     moe_align_block_size,
     moe_sum,
@@ -44,6 +45,7 @@ __all__ = [
     "w8a8_mlp",
     "gemm_gate_up_silu",
     "gemm_down",
+    "gemm_down_bf16",
     "gemm_acc_i32",
     "workspace_bytes",
     "sorted_capacity",

@@ -29,6 +29,10 @@ SIGNATURES = {
     "moe_i8_align_workspace_bytes": (c_int64, [c_int64, c_int, c_int]),
     "moe_i8_align_block_size": (c_int, [_P, c_int64, c_int, c_int, _P, c_int64, _P, c_int64, _P, _P, c_int64, _P]),
     "moe_i8_quant_rows": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, c_int, c_int64, _P, _P, _P]),
+    "moe_i8_gemm_down_bf16": (
+        c_int,
+        [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int64, _P, _P],
+    ),
     "moe_i8_scaled_int8_quant": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, _P]),
     "moe_i8_dense_workspace_bytes": (c_int64, [c_int64, c_int, c_int]),
     "moe_i8_w8a8_linear": (c_int, [_P, _P, _P, _P, c_int64, c_int, c_int, _P, c_int64, c_int, _P]),

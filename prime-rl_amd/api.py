@@ -32,6 +32,7 @@ __all__ = [
     "w8a8_mlp",
     "gemm_gate_up_silu",
     "gemm_down",
+    "gemm_down_bf16",
     "gemm_acc_i32",
     "workspace_bytes",
     "sorted_capacity",
@@ -578,6 +579,32 @@ def gemm_down(
             _ptr(h_q), _ptr(a_scale), _ptr(w2), _ptr(w2_scale), _ptr(tw), _ptr(sorted_token_ids),
             _ptr(expert_ids), _ptr(num_tokens_post_padded), P, E, H, I, _block_size(block_size),
             sorted_token_ids.numel(), _ptr(out), _variant(variant), _stream(h_q),
+        )
+    )
+    return out
+
+
+def gemm_down_bf16(
+    act, w2, w2_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded, block_size: int
+) -> torch.Tensor:
+    """The down GEMM of the streaming family with the second ``per_token_quant_int8`` folded in: ``act`` is
+    the bf16 ``[P, I]`` output of the gate_up GEMM; the result equals quantising it and calling ``gemm_down``."""
+    _require_gpu("act", act)
+    _check_routing(sorted_token_ids, expert_ids, num_tokens_post_padded)
+    w2_scale = _check_weights("w2", w2, w2_scale)
+    E, H, I = w2.shape
+    if act.dtype != torch.bfloat16 or act.dim() != 2 or act.shape[1] != I:
+        raise ValueError("act must be bfloat16 [P, I]")
+    P = act.shape[0]
+    tw = topk_weights.reshape(-1)
+    if tw.dtype != torch.float32 or tw.numel() != P:
+        raise ValueError("topk_weights must be float32 with one entry per pair")
+    out = torch.empty((P, H), dtype=torch.bfloat16, device=act.device)
+    _abi.check(
+        _abi.load().moe_i8_gemm_down_bf16(
+            _ptr(act), _ptr(w2), _ptr(w2_scale), _ptr(tw), _ptr(sorted_token_ids), _ptr(expert_ids),
+            _ptr(num_tokens_post_padded), P, E, H, I, _block_size(block_size), sorted_token_ids.numel(), _ptr(out),
+            _stream(act),
         )
     )
     return out

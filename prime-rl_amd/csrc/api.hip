@@ -48,22 +48,51 @@ int check_gemm_common(const void* a_q, const void* w, const int32_t* sorted, con
   return MOE_I8_OK;
 }
 
-int run_gemm(const moe_i8::GemmArgs& g, int variant, hipStream_t stream) {
-  if (g.num_pairs == 0) return MOE_I8_OK;
-  bool tile;
+// Which family a launch goes to; -1 with the error set if the tile family was demanded for a shape
+// it does not handle.
+int picks_tile(const moe_i8::GemmArgs& g, int variant) {
   if (variant == MOE_I8_GEMM_TILE) {
     if (!moe_i8::gemm_tile_supports(g))
-      return fail(MOE_I8_EUNSUPPORTED, "tile GEMM does not support this shape");
-    tile = true;
-  } else if (variant == MOE_I8_GEMM_STREAM) {
-    tile = false;
-  } else {
-    // Measured crossover on the Qwen3-30B-A3B shape: the streaming family wins while a block holds
-    // one 16-row sub-tile (about 8 routed rows per expert), the LDS-tiled family from about 16 up.
-    tile = moe_i8::gemm_tile_supports(g) && g.num_pairs > (int64_t)12 * g.num_experts;
+      return fail(MOE_I8_EUNSUPPORTED, "tile GEMM does not support this shape"), -1;
+    return 1;
   }
+  if (variant == MOE_I8_GEMM_STREAM) return 0;
+  // Measured crossover on the Qwen3-30B-A3B shape: the streaming family wins while a block holds
+  // one 16-row sub-tile (about 8 routed rows per expert), the LDS-tiled family from about 16 up.
+  return moe_i8::gemm_tile_supports(g) && g.num_pairs > (int64_t)12 * g.num_experts;
+}
+
+int run_gemm(const moe_i8::GemmArgs& g, int variant, hipStream_t stream) {
+  if (g.num_pairs == 0) return MOE_I8_OK;
+  const int tile = picks_tile(g, variant);
+  if (tile < 0) return MOE_I8_EUNSUPPORTED;
   return check_launch(tile ? moe_i8::launch_gemm_tile(g, stream) : moe_i8::launch_gemm_stream(g, stream),
                       tile ? "gemm_tile" : "gemm_stream");
+}
+
+moe_i8::GemmArgs down_args(const int8_t* h_q, const float* a_scale, const int8_t* w2, const float* w2_scale,
+                           const float* topk_weights, const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                           const int32_t* num_tokens_post_padded, int64_t num_pairs, int num_experts, int hidden,
+                           int inter, int block_size, int64_t sorted_cap, void* out) {
+  moe_i8::GemmArgs g{};
+  g.mode = moe_i8::kDown;
+  g.a_q = h_q;
+  g.a_scale = a_scale;
+  g.w = w2;
+  g.w_scale = w2_scale;
+  g.row_weight = topk_weights;
+  g.sorted_token_ids = sorted_token_ids;
+  g.expert_ids = expert_ids;
+  g.num_tokens_post_padded = num_tokens_post_padded;
+  g.num_pairs = num_pairs;
+  g.row_div = 1;
+  g.num_experts = num_experts;
+  g.n = hidden;
+  g.k = inter;
+  g.block_size = block_size;
+  g.sorted_cap = sorted_cap;
+  g.out = out;
+  return g;
 }
 
 }  // namespace
@@ -294,25 +323,29 @@ int moe_i8_gemm_down(const int8_t* h_q, const float* a_scale, const int8_t* w2,
     return rc;
   if (!a_scale || !w2_scale) return fail(MOE_I8_EINVAL, "null scale pointer");
   if (!aligned16(w2_scale)) return fail(MOE_I8_EINVAL, "w2_scale must be 16-byte aligned");
-  moe_i8::GemmArgs g{};
-  g.mode = moe_i8::kDown;
-  g.a_q = h_q;
-  g.a_scale = a_scale;
-  g.w = w2;
-  g.w_scale = w2_scale;
-  g.row_weight = topk_weights;
-  g.sorted_token_ids = sorted_token_ids;
-  g.expert_ids = expert_ids;
-  g.num_tokens_post_padded = num_tokens_post_padded;
-  g.num_pairs = num_pairs;
-  g.row_div = 1;
-  g.num_experts = num_experts;
-  g.n = hidden;
-  g.k = inter;
-  g.block_size = block_size;
-  g.sorted_cap = sorted_cap;
-  g.out = out;
-  return run_gemm(g, variant, static_cast<hipStream_t>(stream));
+  return run_gemm(down_args(h_q, a_scale, w2, w2_scale, topk_weights, sorted_token_ids, expert_ids,
+                            num_tokens_post_padded, num_pairs, num_experts, hidden, inter, block_size, sorted_cap,
+                            out),
+                  variant, static_cast<hipStream_t>(stream));
+}
+
+int moe_i8_gemm_down_bf16(const void* act, const int8_t* w2, const float* w2_scale, const float* topk_weights,
+                          const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                          const int32_t* num_tokens_post_padded, int64_t num_pairs, int num_experts, int hidden,
+                          int inter, int block_size, int64_t sorted_cap, void* out, void* stream) {
+  if (num_pairs == 0) return MOE_I8_OK;
+  if (int rc = check_gemm_common(act, w2, sorted_token_ids, expert_ids, num_tokens_post_padded, out, num_pairs,
+                                 num_experts, hidden, inter, block_size, sorted_cap, MOE_I8_GEMM_STREAM))
+    return rc;
+  if (!w2_scale) return fail(MOE_I8_EINVAL, "null scale pointer");
+  if (!aligned16(w2_scale)) return fail(MOE_I8_EINVAL, "w2_scale must be 16-byte aligned");
+  if (!moe_i8::gemm_stream_fuses_quant(inter))
+    return fail(MOE_I8_EUNSUPPORTED, "inter (%d) is too long for the GEMM that quantises its own activations", inter);
+  moe_i8::GemmArgs g = down_args(nullptr, nullptr, w2, w2_scale, topk_weights, sorted_token_ids, expert_ids,
+                                 num_tokens_post_padded, num_pairs, num_experts, hidden, inter, block_size,
+                                 sorted_cap, out);
+  g.a_bf16 = static_cast<const uint16_t*>(act);
+  return check_launch(moe_i8::launch_gemm_stream(g, static_cast<hipStream_t>(stream)), "gemm_stream");
 }
 
 int moe_i8_gemm_acc_i32(const int8_t* a_q, const int8_t* w, const int32_t* sorted_token_ids,
@@ -465,11 +498,24 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
   if (int rc = moe_i8_gemm_gate_up_silu(x_q, a1, w1, w1_scale, sorted, eids, npp, p, top_k, num_experts,
                                         hidden_size, inter, block_size, c.cap, act, variant, stream))
     return rc;
-  if (int rc = moe_i8_quant_rows(act, MOE_I8_DTYPE_BF16, p, inter, inter, nullptr, 1, p, act_q, a2, stream))
-    return rc;
-  if (int rc = moe_i8_gemm_down(act_q, a2, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
-                                hidden_size, inter, block_size, c.cap, down, variant, stream))
-    return rc;
+  // Very few rows per expert (decode): the streaming down GEMM quantises its activations itself, one
+  // launch less.  Every workgroup of a block repeats that quantisation, so from about four rows
+  // per expert on (measured) the separate launch is the cheaper one again.
+  const moe_i8::GemmArgs dg = down_args(act_q, a2, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
+                                        hidden_size, inter, block_size, c.cap, down);
+  const int down_tile = picks_tile(dg, variant);
+  if (down_tile < 0) return MOE_I8_EUNSUPPORTED;
+  if (!down_tile && moe_i8::gemm_stream_fuses_quant(inter) && p <= (int64_t)3 * num_experts) {
+    if (int rc = moe_i8_gemm_down_bf16(act, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
+                                       hidden_size, inter, block_size, c.cap, down, stream))
+      return rc;
+  } else {
+    if (int rc = moe_i8_quant_rows(act, MOE_I8_DTYPE_BF16, p, inter, inter, nullptr, 1, p, act_q, a2, stream))
+      return rc;
+    if (int rc = moe_i8_gemm_down(act_q, a2, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
+                                  hidden_size, inter, block_size, c.cap, down, variant, stream))
+      return rc;
+  }
   return moe_i8_sum(down, out, m, top_k, hidden_size, stream);
 }
 

@@ -170,6 +170,7 @@ enum GemmMode { kGateUpSilu = 0, kDown = 1, kAccI32 = 2 };
 
 struct GemmArgs {
   int mode;
+  const uint16_t* a_bf16 = nullptr;  // down, streaming family only: bf16 activations [P, K] quantised in the kernel
   const int8_t* a_q;      // [*, K] activations (int8)
   const float* a_scale;   // per activation row
   const int8_t* w;        // [E, N, K]
@@ -188,6 +189,7 @@ struct GemmArgs {
   void* out;  // bf16 [P, I] | bf16 [P, H] | int32 [P, N]
 };
 hipError_t launch_gemm_stream(const GemmArgs& a, hipStream_t stream);
+bool gemm_stream_fuses_quant(int k);  // the down GEMM can quantise bf16 activations of this length itself
 hipError_t launch_gemm_tile(const GemmArgs& a, hipStream_t stream);
 bool gemm_tile_supports(const GemmArgs& a);
 

@@ -21,6 +21,7 @@
 // finds them in L2); sub-tiles that hold only padding are skipped (valid rows are a prefix of the
 // block).  Blocks with many rows belong to the LDS-tiled family.
 #include "common.hpp"
+#include "quant_body.hpp"
 
 namespace moe_i8 {
 namespace {
@@ -35,8 +36,14 @@ constexpr int kWinBytes = 256;                              // bytes of every we
 constexpr int kWinSteps = kWinBytes / kStepK;               // MFMA steps per window
 constexpr int kWinLoads = kTiles * 16 * kWinBytes / 1024;   // 1 KB wave-level loads per window
 constexpr int kWaveLds = kTiles * 16 * kWinBytes;           // LDS bytes per wavefront
+// Down GEMM that quantises its own activations: the 16 rows of a sub-tile are quantised from bf16
+// into this LDS area by the workgroup (rows padded by 16 bytes so that the 16 rows of one operand
+// read fall on different banks), reduction length limited accordingly.
+constexpr int kFusedMaxK = 1024;
+constexpr int kFusedRowPad = 16;
 
 struct StreamParams {
+  const uint16_t* a_bf16;  // fused-quantisation variant: bf16 activations [P, K] instead of a_q / a_scale
   const int8_t* a_q;
   const float* a_scale;
   const int8_t* w;
@@ -83,9 +90,15 @@ __device__ __forceinline__ void pair_rows(const StreamParams& p, int q, int (&wr
 
 // `count_valid`: first pass over a block; the number of valid rows of the block is counted here,
 // after the first weight window has been requested, and returned.
-template <int MODE, int NS>
+//
+// kFused: the activations arrive as bf16; the workgroup quantises the 16 rows of the sub-tile into
+// `a_lds` (int8) and `s_lds` (row scales) with the arithmetic of the stand-alone quantiser and the
+// operand reads come from there.  Every wavefront of the workgroup must call this, also those with
+// no weight rows left (`npairs` == 0): they take part in the quantisation and its two barriers.
+template <int MODE, int NS, bool kFused>
 __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e, int sub0, int first_pair,
-                                           int npairs, char* wave_lds, bool count_valid) {
+                                           int npairs, char* wave_lds, bool count_valid, char* a_lds,
+                                           float* s_lds) {
   const int lane = lane_id();
   const int col = lane & 15;  // token slot inside a sub-tile / weight row inside a tile
   const int grp = lane >> 4;  // which 16 reduction bytes of each step; which 4 output channels
@@ -100,25 +113,34 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
   const int rd_base = col * kWinBytes + ((grp ^ col) * 16);             // ^ u * 64, + t * 4096
 
   // The wavefront walks windows (pair 0, k 0), (pair 0, k 256), ..., (pair 1, k 0), ... ; `fq`/`fk`
-  // track the window being fetched, `cq`/`ck` the one being consumed.
-  int fq = 0, fk = 0;
+  // track the window whose weights are being fetched (`fk` also the one whose activation rows are),
+  // `cq`/`ck` the one being consumed.
+  int fq = 0, wk = 0, fk = 0;
   auto fetch_weights = [&](Window<NS>& win) {
     int wrow[kTiles];
     bool wok[kTiles];
     pair_rows<MODE>(p, first_pair + fq, wrow, wok);
-    const bool chunk_in = fk + ld_chunk * 16 < K;  // only the last window of a ragged K is partial
+    const bool chunk_in = wk + ld_chunk * 16 < K;  // only the last window of a ragged K is partial
 #pragma unroll
     for (int j = 0; j < kWinLoads; ++j) {
-      const int8_t* src = wbase + (int64_t)(wrow[j / 4] + 4 * (j % 4)) * K + fk;
+      const int8_t* src = wbase + (int64_t)(wrow[j / 4] + 4 * (j % 4)) * K + wk;
       win.w[j] = chunk_in ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src)) : v4i{0, 0, 0, 0};
+    }
+    wk += kWinBytes;
+    if (wk >= K) {
+      wk = 0;
+      ++fq;
     }
   };
 
-  // The weights of the first window depend on nothing but the expert of the block: they are
-  // requested from HBM before the chain of dependent reads (row list -> token -> activation row)
-  // that the rest of the set-up is.
+  // The weights of the first two windows depend on nothing but the expert of the block: they are
+  // requested from HBM before the chain of dependent reads (row list -> token -> activation row,
+  // or the quantisation of the rows) that the rest of the set-up is.
+  const int nwin = (K + kWinBytes - 1) / kWinBytes;
+  const int total = npairs * nwin;
   Window<NS> w0, w1;
-  fetch_weights(w0);
+  if (total > 0) fetch_weights(w0);
+  if (total > 1) fetch_weights(w1);
 
   int nvalid = 0;
   if (count_valid) {
@@ -129,6 +151,39 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
     }
   }
 
+  if constexpr (kFused) {
+    static_assert(NS == 1, "one sub-tile per pass");
+    const int wave = threadIdx.x / kWave;
+    const int row_bytes = K + kFusedRowPad;
+    __syncthreads();  // the previous pass is done reading a_lds
+#pragma unroll
+    for (int i = 0; i < kSub / kWaves; ++i) {
+      const int r = wave * (kSub / kWaves) + i;
+      const int32_t t = p.sorted_ids[(int64_t)blk * p.B + sub0 * kSub + r];  // wave-uniform
+      if (t < 0 || t >= p.P) continue;
+      const uint4* in = reinterpret_cast<const uint4*>(p.a_bf16 + (int64_t)t * K);
+      const int nvec = K / kQuantVec;
+      uint4 v[kFusedMaxK / kQuantVec / kWave];
+      float m = 0.0f;
+#pragma unroll
+      for (int c = 0; c < kFusedMaxK / kQuantVec / kWave; ++c) {
+        const int idx = lane + c * kWave;
+        v[c] = idx < nvec ? in[idx] : make_uint4(0u, 0u, 0u, 0u);
+        m = fmaxf(m, absmax8(v[c]));
+      }
+      const float absmax = fmaxf(wave_max(m), 1e-10f);
+      const float inv = 127.0f / absmax;
+      if (lane == 0) s_lds[r] = absmax / 127.0f;
+#pragma unroll
+      for (int c = 0; c < kFusedMaxK / kQuantVec / kWave; ++c) {
+        const int idx = lane + c * kWave;
+        if (idx < nvec) *reinterpret_cast<uint2*>(a_lds + r * row_bytes + idx * 8) = quant8(v[c], inv);
+      }
+    }
+    __syncthreads();
+    if (npairs == 0) return nvalid;
+  }
+
   int32_t tok[NS];
   bool tok_ok[NS];
   const int8_t* ap[NS];
@@ -137,8 +192,9 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
     tok[s] = p.sorted_ids[(int64_t)blk * p.B + (sub0 + s) * kSub + col];
     tok_ok[s] = tok[s] >= 0 && tok[s] < p.P;
     const int64_t arow = tok_ok[s] ? tok[s] / p.row_div : 0;
-    ap[s] = p.a_q + arow * K + grp * 16;
+    ap[s] = kFused ? nullptr : p.a_q + arow * K + grp * 16;
   }
+  const char* a_row = a_lds + col * (K + kFusedRowPad) + grp * 16;  // fused: this lane's operand row
 
   v4i acc[kTiles][NS];
 #pragma unroll
@@ -150,14 +206,16 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
 #pragma unroll
     for (int s = 0; s < NS; ++s)
 #pragma unroll
-      for (int u = 0; u < kWinSteps; ++u)
-        win.a[s][u] = fk + u * kStepK < K ? *reinterpret_cast<const v4i*>(ap[s] + fk + u * kStepK)
-                                           : v4i{0, 0, 0, 0};
+      for (int u = 0; u < kWinSteps; ++u) {
+        if constexpr (kFused)
+          win.a[s][u] = fk + u * kStepK < K ? *reinterpret_cast<const v4i*>(a_row + fk + u * kStepK)
+                                             : v4i{0, 0, 0, 0};
+        else
+          win.a[s][u] = fk + u * kStepK < K ? *reinterpret_cast<const v4i*>(ap[s] + fk + u * kStepK)
+                                             : v4i{0, 0, 0, 0};
+      }
     fk += kWinBytes;
-    if (fk >= K) {
-      fk = 0;
-      ++fq;
-    }
+    if (fk >= K) fk = 0;
   };
   auto fetch = [&](Window<NS>& win) {
     fetch_weights(win);
@@ -182,7 +240,7 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
 #pragma unroll
       for (int s = 0; s < NS; ++s) {
         if (!tok_ok[s]) continue;
-        const float as = p.a_scale[tok[s] / p.row_div];
+        const float as = kFused ? s_lds[col] : p.a_scale[tok[s] / p.row_div];
         const float rw = p.row_weight ? p.row_weight[tok[s]] : 1.0f;
 #pragma unroll
         for (int t = 0; t < kTiles; ++t) {
@@ -239,11 +297,12 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
     }
   };
 
-  const int nwin = (K + kWinBytes - 1) / kWinBytes;
-  const int total = npairs * nwin;
   fetch_rows(w0);
   for (int i = 0; i < total; i += 2) {
-    if (i + 1 < total) fetch(w1);
+    if (i + 1 < total) {
+      if (i > 0) fetch_weights(w1);  // the weights of window 1 were requested up front
+      fetch_rows(w1);
+    }
     consume(w0);
     if (i + 1 >= total) break;
     if (i + 2 < total) fetch(w0);
@@ -253,32 +312,37 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
 }
 
 // grid.x: groups of kWaves wavefronts along the weight rows; grid.y: 64-row (B-row) blocks.
-template <int MODE>
+template <int MODE, bool kFused>
 __global__ __launch_bounds__(kThreads, 3) void gemm_stream_kernel(StreamParams p) {
   __shared__ __align__(16) char lds[kWaves * kWaveLds];
+  __shared__ __align__(16) char a_lds[kFused ? kSub * (kFusedMaxK + kFusedRowPad) : 16];
+  __shared__ float s_lds[kSub];
   const int blk = blockIdx.y;
   const int npp = *p.npp;
   if ((int64_t)blk * p.B >= npp) return;
   const int e = p.expert_ids[blk];
   if (e < 0 || e >= p.E) return;
-  const int lane = lane_id();
   const int total_pairs = MODE == kGateUpSilu ? p.N / 2 / 16 : (p.N / 16 + kTiles - 1) / kTiles;
   const int first_pair = (blockIdx.x * kWaves + threadIdx.x / kWave) * p.pairs_per_wave;
-  if (first_pair >= total_pairs) return;
-  const int npairs = total_pairs - first_pair < p.pairs_per_wave ? total_pairs - first_pair : p.pairs_per_wave;
+  // a wavefront past the last weight rows leaves, unless the workgroup needs it for the quantisation
+  if (!kFused && first_pair >= total_pairs) return;
+  const int left = total_pairs - first_pair;
+  const int npairs = left < 0 ? 0 : left < p.pairs_per_wave ? left : p.pairs_per_wave;
 
   // Valid rows are a prefix of the block (at least one, the block is in use): the first pass counts
   // them to know how many sub-tiles there are.
   char* wave_lds = lds + (threadIdx.x / kWave) * kWaveLds;
-  const int nvalid = stream_pass<MODE, kGroup>(p, blk, e, 0, first_pair, npairs, wave_lds, true);
+  const int nvalid =
+      stream_pass<MODE, kGroup, kFused>(p, blk, e, 0, first_pair, npairs, wave_lds, true, a_lds, s_lds);
   const int nsub = (nvalid + kSub - 1) / kSub;
   for (int sub0 = kGroup; sub0 < nsub; sub0 += kGroup)
-    stream_pass<MODE, kGroup>(p, blk, e, sub0, first_pair, npairs, wave_lds, false);
+    stream_pass<MODE, kGroup, kFused>(p, blk, e, sub0, first_pair, npairs, wave_lds, false, a_lds, s_lds);
 }
 
-template <int MODE>
+template <int MODE, bool kFused = false>
 hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   StreamParams p;
+  p.a_bf16 = a.a_bf16;
   p.a_q = a.a_q;
   p.a_scale = a.a_scale;
   p.w = a.w;
@@ -304,16 +368,23 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   if (blocks == 0 || waves == 0) return hipSuccess;
   if (blocks > 65535) return hipErrorInvalidValue;
   const dim3 grid((unsigned)((waves + kWaves - 1) / kWaves), (unsigned)blocks);
-  hipLaunchKernelGGL(gemm_stream_kernel<MODE>, grid, dim3(kThreads), 0, stream, p);
+  hipLaunchKernelGGL((gemm_stream_kernel<MODE, kFused>), grid, dim3(kThreads), 0, stream, p);
   return hipGetLastError();
 }
 
 }  // namespace
 
+bool gemm_stream_fuses_quant(int k) { return k <= kFusedMaxK; }
+
 hipError_t launch_gemm_stream(const GemmArgs& a, hipStream_t stream) {
   switch (a.mode) {
     case kGateUpSilu: return launch_mode<kGateUpSilu>(a, stream);
-    case kDown: return launch_mode<kDown>(a, stream);
+    case kDown:
+      if (a.a_bf16) {
+        if (a.k > kFusedMaxK || a.row_div != 1) return hipErrorInvalidValue;
+        return launch_mode<kDown, true>(a, stream);
+      }
+      return launch_mode<kDown>(a, stream);
     case kAccI32: return launch_mode<kAccI32>(a, stream);
     default: return hipErrorInvalidValue;
   }

@@ -89,6 +89,26 @@ def test_down_gemm_epilogue_bit_exact(pra, oracle, variant, E, k, H, I, M, B):
     assert torch.equal(out.cpu(), want), int((out.cpu() != want).sum())
 
 
+@pytest.mark.parametrize("E,k,H,I,M,B", SHAPES + [(8, 2, 256, 1024, 130, 64), (8, 2, 128, 1000 // 64 * 64, 70, 16)])
+def test_down_gemm_that_quantises_its_own_activations(pra, oracle, E, k, H, I, M, B):
+    # bf16 activations in, the second per-token quantisation inside the kernel: the same bits as
+    # quantise-then-GEMM (and so as the oracle)
+    inp, st = _problem(oracle, E, k, H, I, M, seed=E + M + 3, B=B)
+    s, e, npp = _routing_on_gpu(pra, inp, B)
+    args = (st["cache2"].to(DEV), inp.w2.to(DEV), inp.w2_scale.to(DEV), inp.topk_weights.to(DEV), s, e, npp, B)
+    if I > 1024:
+        with pytest.raises(pra._abi.MoeI8Error) as info:
+            pra.gemm_down_bf16(*args)
+        assert info.value.code == pra._abi.EUNSUPPORTED
+        return
+    out = pra.gemm_down_bf16(*args)
+    want = st["cache3"].reshape(M * k, H)
+    assert torch.equal(out.cpu(), want), int((out.cpu() != want).sum())
+    two_step = pra.gemm_down(*pra.per_token_quant_int8(st["cache2"].to(DEV)), inp.w2.to(DEV), inp.w2_scale.to(DEV),
+                             inp.topk_weights.to(DEV), s, e, npp, B, "stream")
+    assert torch.equal(out, two_step)
+
+
 @pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("E,k,H,I,M,B", SHAPES)
 def test_gate_up_silu_within_bf16_rounding(pra, oracle, variant, E, k, H, I, M, B):
