@@ -1,0 +1,74 @@
+"""GPU parity on seeded random problem shapes: both GEMM families' int32 accumulators and the down epilogue
+bit-exact, the whole layer within tolerance.  The shapes vary every size the index arithmetic depends on
+(experts, top-k, hidden and intermediate sizes that are and are not multiples of the tile sizes, block size,
+rows per expert from none to several tiles, skewed routing)."""
+
+import random
+
+import pytest
+import torch
+
+from _util import inputs_mod, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _cases():
+    rng = random.Random(1234)
+    cases = []
+    for i in range(120):
+        E = rng.choice([1, 2, 3, 5, 8, 16, 24, 40, 64])
+        k = rng.choice([1, 2, 3, 4, 6, 8])
+        k = min(k, E)
+        H = 64 * rng.choice([1, 2, 3, 4, 5, 8, 9, 16, 22, 32])
+        I = 64 * rng.choice([1, 2, 3, 4, 6, 7, 11, 12])
+        B = rng.choice([16, 32, 64, 64, 128])
+        rows_per_expert = rng.choice([0.3, 2, 9, 17, 40, 64, 70, 130, 257, 300, 700, 1500])
+        M = max(1, int(rows_per_expert * E / k))
+        if M * k * I * H > 1.5e10:  # keep the CPU oracle in seconds
+            M = max(1, int(1.5e10 / (k * I * H)))
+        routing = rng.choice(["softmax", "softmax", "zipf"])
+        cases.append((i, E, k, H, I, M, B, routing))
+    return cases
+
+
+@pytest.mark.parametrize("case", _cases(), ids=lambda c: "n{}-E{}k{}H{}I{}M{}B{}-{}".format(*c))
+def test_random_shape(pra, oracle, case):
+    i, E, k, H, I, M, B, routing = case
+    im = inputs_mod()
+    shape = im.LayerShape("r", E=E, k=k, H=H, I=I, routing=routing)
+    inp = im.make_inputs(shape, M, seed=1000 + i)
+    st = oracle.fused_experts_staged(inp.hidden_states, inp.w1, inp.w2, inp.topk_weights, inp.topk_ids,
+                                     inp.w1_scale, inp.w2_scale, B)
+    d = inp.to(DEV)
+    s, e, npp = pra.moe_align_block_size(d.topk_ids, B, E)
+    P = M * k
+    x_q, h_q = st["x_q"].to(DEV), st["h_q"].to(DEV)
+    a2 = st["a2_scale"].to(DEV)
+    ran = 0
+    for variant in ("stream", "tile"):
+        try:
+            acc1 = pra.gemm_acc_i32(x_q, d.w1, s, e, npp, k, B, P, variant)
+            acc2 = pra.gemm_acc_i32(h_q, d.w2, s, e, npp, 1, B, P, variant)
+            down = pra.gemm_down(h_q, a2, d.w2, d.w2_scale, d.topk_weights, s, e, npp, B, variant)
+        except pra._abi.MoeI8Error as exc:
+            if exc.code == pra._abi.EUNSUPPORTED:
+                continue
+            raise
+        ran += 1
+        assert torch.equal(acc1.cpu(), st["acc1"]), (variant, int((acc1.cpu() != st["acc1"]).sum()))
+        assert torch.equal(acc2.cpu(), st["acc2"]), (variant, int((acc2.cpu() != st["acc2"]).sum()))
+        want = st["cache3"].reshape(P, H)
+        assert torch.equal(down.cpu(), want), (variant, int((down.cpu() != want).sum()))
+    assert ran >= 1
+    for variant in ("auto", "tile"):
+        try:
+            out = pra.fused_experts(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, use_int8_w8a8=True,
+                                    per_channel_quant=True, w1_scale=d.w1_scale, w2_scale=d.w2_scale,
+                                    block_size_m=B, gemm_variant=variant)
+        except pra._abi.MoeI8Error as exc:
+            if exc.code == pra._abi.EUNSUPPORTED:
+                continue
+            raise
+        assert rel_err(out, st["out"]) < 1e-2, variant
