@@ -1,12 +1,15 @@
-// Per-token dynamic symmetric int8 quantisation for gfx950, optionally fused with a row gather.
+// Symmetric int8 quantisation for gfx950, one scale per row: activations (per token, optionally
+// fused with a row gather) and weights (per output channel).
 //
-// One 64-lane wavefront owns one output row.  The row is read once with 16-byte loads (8 bf16 per
-// lane per load, all loads issued before the first use), the absolute maximum is reduced across
-// the wavefront with lane shuffles, and 8 int8 per lane are written with 8-byte stores.  HBM
-// traffic is the minimum 2 + 1 bytes per element plus 4 bytes per row.
-//
+// Activations: one 64-lane wavefront owns one output row.  The row is read once with 16-byte loads
+// (8 bf16 per lane per load, all loads issued before the first use), the absolute maximum is
+// reduced across the wavefront with lane permutes, and 8 int8 per lane are written with 8-byte
+// stores.  HBM traffic is the minimum 2 + 1 bytes per element plus 4 bytes per row.
 // Arithmetic (fp32): absmax = max(max|x|, 1e-10); scale = absmax / 127;
-// q = roundf(x * (127 / absmax))  (ties away from zero).
+// q = round(x * (127 / absmax)), ties away from zero (MoE path) or to even (dense path).
+//
+// Weights: scale = max(absmax / 127, 1e-12); q = rint(x / scale); a wavefront walks several
+// consecutive rows with the next rows' loads in flight (see quant_weights_kernel).
 #include "quant_body.hpp"
 
 namespace moe_i8 {
@@ -39,13 +42,8 @@ void launch_quant_rows_mode(const QuantArgs& a, dim3 grid, dim3 block, hipStream
 // wavefront that lives for a single row spends much of its life with nothing outstanding, and
 // short rows need several in flight to cover the HBM latency).  kDepth * VPL = 8 vectors of 16
 // bytes per lane, 8 KB per wavefront.  Loads and stores are nontemporal: every byte is touched once.
-#ifndef MOE_I8_WQ_ROWS
-#define MOE_I8_WQ_ROWS 16
-#endif
-#ifndef MOE_I8_WQ_INFLIGHT
-#define MOE_I8_WQ_INFLIGHT 8
-#endif
-constexpr int kWeightRowsPerWave = MOE_I8_WQ_ROWS;
+constexpr int kWeightRowsPerWave = 16;
+constexpr int kWeightVectorsInFlight = 8;  // 16-byte loads per lane kept in flight
 
 // No branch around the loads (the compiler would wait for everything outstanding at the join):
 // lanes past the end of the row, and rows past the end of the wavefront's share, read the first
@@ -66,7 +64,7 @@ __device__ __forceinline__ uint4 as_uint4(const v4i& v) {
 
 template <int VPL>
 __global__ __launch_bounds__(kThreads) void quant_weights_kernel(QuantArgs a) {
-  constexpr int kDepth = MOE_I8_WQ_INFLIGHT / VPL > 1 ? MOE_I8_WQ_INFLIGHT / VPL : 1;
+  constexpr int kDepth = kWeightVectorsInFlight / VPL > 1 ? kWeightVectorsInFlight / VPL : 1;
   static_assert(kWeightRowsPerWave % kDepth == 0, "ring depth must divide the rows of a wavefront");
   const int lane = lane_id();
   const int64_t wave = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
