@@ -9,6 +9,7 @@ from .api import (  # noqa: F401
     DEFAULT_BLOCK_SIZE_M,
     apply_int8_linear,
     fused_experts,
+    fused_moe,
     fused_topk,
     grouped_topk,
     route_topk,
@@ -31,6 +32,7 @@ from . import api, build, vllm_plugin  # noqa: F401
 
 __all__ = [
     "fused_experts",
+    "fused_moe",
     "moe_align_block_size",
     "per_token_quant_int8",
     "quantize_weights_per_channel",

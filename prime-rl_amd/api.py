@@ -18,6 +18,7 @@ from . import _abi
 
 __all__ = [
     "fused_experts",
+    "fused_moe",
     "moe_align_block_size",
     "per_token_quant_int8",
     "quantize_weights_per_channel",
@@ -738,3 +739,67 @@ def fused_experts(
         )
     )
     return out
+
+
+def fused_moe(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    gating_output: torch.Tensor,
+    topk: int,
+    renormalize: bool,
+    inplace: bool = False,
+    activation: str = "silu",
+    use_grouped_topk: bool = False,
+    num_expert_group: int | None = None,
+    topk_group: int | None = None,
+    custom_routing_function=None,
+    use_int8_w8a8: bool = False,
+    per_channel_quant: bool = False,
+    global_num_experts: int = -1,
+    expert_map: torch.Tensor | None = None,
+    w1_scale: torch.Tensor | None = None,
+    w2_scale: torch.Tensor | None = None,
+    a1_scale: torch.Tensor | None = None,
+    a2_scale: torch.Tensor | None = None,
+    block_shape: list[int] | None = None,
+    *,
+    scoring_func: str = "softmax",
+    routed_scaling_factor: float = 1.0,
+    e_score_correction_bias: torch.Tensor | None = None,
+    routed_experts_out: tuple[torch.Tensor, int] | None = None,
+    block_size_m: int = DEFAULT_BLOCK_SIZE_M,
+    gemm_variant: str | int = "auto",
+    workspace: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """vLLM ``fused_moe``: routing from the router logits (``fused_topk``, or ``grouped_topk`` with
+    ``use_grouped_topk``) followed by ``fused_experts`` — the router launch and the layer's launches on the
+    current stream.  ``gating_output`` must be float32 (the reference runs its router in fp32,
+    ``src/prime_rl/trainer/models/layers/moe.py:262-269``)."""
+    if custom_routing_function is not None:
+        raise NotImplementedError("custom_routing_function is not supported")
+    if gating_output.dtype != torch.float32:
+        gating_output = gating_output.float()
+    if use_grouped_topk:
+        if not num_expert_group or not topk_group:
+            raise ValueError("use_grouped_topk needs num_expert_group and topk_group")
+        topk_weights, topk_ids = grouped_topk(
+            hidden_states, gating_output, topk, renormalize, num_expert_group, topk_group, scoring_func,
+            routed_scaling_factor, e_score_correction_bias, routed_experts_out=routed_experts_out,
+        )
+    else:
+        if scoring_func != "softmax" or e_score_correction_bias is not None or routed_scaling_factor != 1.0:
+            topk_weights, topk_ids = route_topk(
+                gating_output, topk, score_func=scoring_func, renormalize=renormalize,
+                route_scale=routed_scaling_factor, selection_bias=e_score_correction_bias,
+                routed_experts_out=routed_experts_out,
+            )
+        else:
+            topk_weights, topk_ids = fused_topk(hidden_states, gating_output, topk, renormalize,
+                                                routed_experts_out=routed_experts_out)
+    return fused_experts(
+        hidden_states, w1, w2, topk_weights, topk_ids, inplace=inplace, activation=activation,
+        use_int8_w8a8=use_int8_w8a8, per_channel_quant=per_channel_quant, global_num_experts=global_num_experts,
+        expert_map=expert_map, w1_scale=w1_scale, w2_scale=w2_scale, a1_scale=a1_scale, a2_scale=a2_scale,
+        block_shape=block_shape, block_size_m=block_size_m, gemm_variant=gemm_variant, workspace=workspace,
+    )

@@ -171,3 +171,35 @@ def test_router_feeds_the_layer(pra, oracle):
     ref = oracle.fused_experts(inp.hidden_states, inp.w1, inp.w2, wo, ido, inp.w1_scale, inp.w2_scale)
     from _util import rel_err
     assert rel_err(out.cpu(), ref) < 1e-2
+
+
+def test_fused_moe_from_router_logits(pra, oracle):
+    # vLLM fused_moe = routing + experts: softmax router on the toy shape, grouped sigmoid router on a
+    # DeepSeek-like one, both against oracle router -> oracle layer
+    from _util import rel_err
+
+    im = inputs_mod()
+    shape = im.SHAPES["toy"]
+    inp = im.make_inputs(shape, 33, seed=4)
+    d = inp.to(DEV)
+    logits = torch.randn(33, shape.E, generator=torch.Generator().manual_seed(6))
+    record = torch.zeros(33, 2, shape.k, dtype=torch.uint8, device=DEV)
+    out = pra.fused_moe(d.hidden_states, d.w1, d.w2, logits.to(DEV), shape.k, True, use_int8_w8a8=True,
+                        per_channel_quant=True, w1_scale=d.w1_scale, w2_scale=d.w2_scale,
+                        routed_experts_out=(record, 1))
+    wo, ido = oracle.route_topk(logits, shape.k)
+    ref = oracle.fused_experts(inp.hidden_states, inp.w1, inp.w2, wo, ido, inp.w1_scale, inp.w2_scale)
+    assert rel_err(out.cpu(), ref) < 1e-2
+    assert torch.equal(record[:, 1, :].cpu().to(torch.int32), ido) and int(record[:, 0, :].abs().sum()) == 0
+    gshape = im.LayerShape("g", E=64, k=6, H=256, I=128)
+    ginp = im.make_inputs(gshape, 21, seed=5)
+    gd = ginp.to(DEV)
+    glogits = torch.randn(21, 64, generator=torch.Generator().manual_seed(7))
+    bias = torch.randn(64, generator=torch.Generator().manual_seed(8)) * 0.1
+    out = pra.fused_moe(gd.hidden_states, gd.w1, gd.w2, glogits.to(DEV), 6, True, use_grouped_topk=True,
+                        num_expert_group=8, topk_group=3, use_int8_w8a8=True, per_channel_quant=True,
+                        w1_scale=gd.w1_scale, w2_scale=gd.w2_scale, scoring_func="sigmoid",
+                        routed_scaling_factor=2.5, e_score_correction_bias=bias.to(DEV))
+    wo, ido = oracle.grouped_topk(glogits, bias, 6, 8, 3, True, 2.5)
+    ref = oracle.fused_experts(ginp.hidden_states, ginp.w1, ginp.w2, wo, ido, ginp.w1_scale, ginp.w2_scale)
+    assert rel_err(out.cpu(), ref) < 1e-2
