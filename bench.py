@@ -96,6 +96,69 @@ def time_gate_up_kernel(pkg, torch, shape, dev, weights, steps: int, warmup: int
     return sum(a.elapsed_time(b) for a, b in zip(starts, stops)) / steps * 1e-3
 
 
+def time_stages(pkg, torch, shape, dev, weights, steps: int, warmup: int, variant: str) -> list:
+    """Every launch of the layer on its own: direct C-ABI calls into preallocated buffers, an event pair per
+    call on the launch stream, with the algorithmic bytes / int8 ops of that launch and the fraction of the
+    roofline that bounds it.  (A launch that does almost nothing still reads about 4 us.)"""
+    abi = pkg._abi
+    lib = abi.load()
+    M, k = dev.topk_ids.shape
+    P, H, I, E = M * k, shape.H, shape.I, shape.E_total
+    n_act = int(torch.unique(dev.topk_ids).numel())
+    x_q, a1 = pkg.per_token_quant_int8(dev.hidden_states)
+    s, e, npp = pkg.moe_align_block_size(dev.topk_ids, 64, E)
+    w1, w2, s1, s2 = weights[0]
+    act = pkg.gemm_gate_up_silu(x_q, a1, w1, s1, s, e, npp, k, 64, P, variant)
+    h_q, a2 = pkg.per_token_quant_int8(act)
+    down = pkg.gemm_down(h_q, a2, w2, s2, dev.topk_weights, s, e, npp, 64, variant)
+    out = torch.empty_like(dev.hidden_states)
+    ws_bytes = lib.moe_i8_align_workspace_bytes(P, E, 64)
+    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device="cuda:0")
+    ids32 = dev.topk_ids.to(torch.int32).contiguous()
+    tw = dev.topk_weights.reshape(-1).contiguous()
+    stream = torch.cuda.current_stream().cuda_stream
+    v = {"auto": abi.GEMM_AUTO, "stream": abi.GEMM_STREAM, "tile": abi.GEMM_TILE}[variant]
+    n = len(weights)
+    p_ = lambda t: t.data_ptr()
+    stages = [
+        ("quant input",
+         lambda i: lib.moe_i8_quant_rows(p_(dev.hidden_states), abi.DTYPE_BF16, M, H, H, None, 1, M, p_(x_q), p_(a1), stream),
+         3 * M * H + 4 * M, 0),
+        ("moe_align",
+         lambda i: lib.moe_i8_align_block_size(p_(ids32), P, E, 64, p_(s), s.numel(), p_(e), e.numel(), p_(npp), p_(ws),
+                                               ws.numel(), stream),
+         8 * P, 0),
+        ("gemm gate_up + SiLU*mul",
+         lambda i: lib.moe_i8_gemm_gate_up_silu(p_(x_q), p_(a1), p_(weights[i % n][0]), p_(weights[i % n][2]), p_(s), p_(e),
+                                                p_(npp), P, k, E, H, I, 64, s.numel(), p_(act), v, stream),
+         n_act * (2 * I * H + 8 * I) + M * H + 4 * M + 2 * P * I + 4 * P, 4 * P * I * H),
+        ("quant activations",
+         lambda i: lib.moe_i8_quant_rows(p_(act), abi.DTYPE_BF16, P, I, I, None, 1, P, p_(h_q), p_(a2), stream),
+         3 * P * I + 4 * P, 0),
+        ("gemm down * routed weight",
+         lambda i: lib.moe_i8_gemm_down(p_(h_q), p_(a2), p_(weights[i % n][1]), p_(weights[i % n][3]), p_(tw), p_(s), p_(e),
+                                        p_(npp), P, E, H, I, 64, s.numel(), p_(down), v, stream),
+         n_act * (H * I + 4 * H) + P * I + 8 * P + 2 * P * H, 2 * P * I * H),
+        ("moe_sum", lambda i: lib.moe_i8_sum(p_(down), p_(out), M, k, H, stream), 2 * (k + 1) * M * H, 0),
+    ]
+    result = []
+    for name, fn, nbytes, ops in stages:
+        for i in range(warmup):
+            abi.check(fn(i))
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(pairs):
+            a.record()
+            fn(i)
+            b.record()
+        torch.cuda.synchronize()
+        t = sum(a.elapsed_time(b) for a, b in pairs) / steps * 1e-3
+        hbm, mfma = nbytes / t / PEAK_HBM_BPS, ops / t / PEAK_INT8_OPS
+        result.append({"stage": name, "us": t * 1e6, "bytes": nbytes, "int8_ops": ops, "hbm_frac": hbm,
+                       "mfma_frac": mfma, "bound": "mfma" if mfma > hbm else "hbm"})
+    return result
+
+
 def gate_up_work(shape, M: int, topk_ids):
     """Algorithmic work of one gate_up GEMM launch: int8 ops, and HBM bytes (weights and channel
     scales of the routed-to experts, int8 activations and their scales in, bf16 activations out)."""
@@ -264,6 +327,9 @@ def main() -> int:
             "layer_hbm_frac": bytes_layer / t_layer / PEAK_HBM_BPS,
             "roofline": roof,
         }
+        if M == args.m:
+            point["stages"] = time_stages(pkg, torch, shape, dev, weights, max(args.steps // 2, 1),
+                                          max(args.warmup // 2, 1), args.variant)
         sweep.append(point)
         if M == args.m:
             headline, base_headline = point, base
