@@ -58,8 +58,8 @@ int picks_tile(const moe_i8::GemmArgs& g, int variant) {
   }
   if (variant == MOE_I8_GEMM_STREAM) return 0;
   // Measured crossover on the Qwen3-30B-A3B shape: the streaming family wins while a block holds
-  // one 16-row sub-tile (about 8 routed rows per expert), the LDS-tiled family from about 16 up.
-  return moe_i8::gemm_tile_supports(g) && g.num_pairs > (int64_t)12 * g.num_experts;
+  // one or two 16-row sub-tiles (up to about 24 routed rows per expert), the LDS-tiled family beyond.
+  return moe_i8::gemm_tile_supports(g) && g.num_pairs > (int64_t)24 * g.num_experts;
 }
 
 int run_gemm(const moe_i8::GemmArgs& g, int variant, hipStream_t stream) {

@@ -29,7 +29,11 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
 constexpr int kSub = 16;      // token rows per sub-tile (MFMA N)
-constexpr int kGroup = 1;     // sub-tiles processed per pass over the weights
+// Sub-tiles processed per pass over the weights: one while blocks rarely hold more than 16 rows (12
+// wavefronts fit a CU), two beyond (the second sub-tile reuses the weights in registers instead of
+// a second pass; the larger register set leaves 8 wavefronts per CU).  Measured crossover on the
+// Qwen3-30B-A3B shape: about 10 routed rows per expert.
+constexpr int kPairRowsPerExpert = 10;
 constexpr int kStepK = 64;    // reduction bytes per MFMA
 constexpr int kTiles = 2;     // 16-row weight tiles per wavefront
 constexpr int kWinBytes = 256;                              // bytes of every weight row per window
@@ -189,7 +193,8 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
   const int8_t* ap[NS];
 #pragma unroll
   for (int s = 0; s < NS; ++s) {
-    tok[s] = p.sorted_ids[(int64_t)blk * p.B + (sub0 + s) * kSub + col];
+    const int slot = (sub0 + s) * kSub + col;  // a second sub-tile may lie past the end of a small block
+    tok[s] = slot < p.B ? p.sorted_ids[(int64_t)blk * p.B + slot] : -1;
     tok_ok[s] = tok[s] >= 0 && tok[s] < p.P;
     const int64_t arow = tok_ok[s] ? tok[s] / p.row_div : 0;
     ap[s] = kFused ? nullptr : p.a_q + arow * K + grp * 16;
@@ -312,8 +317,9 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
 }
 
 // grid.x: groups of kWaves wavefronts along the weight rows; grid.y: 64-row (B-row) blocks.
-template <int MODE, bool kFused>
-__global__ __launch_bounds__(kThreads, 3) void gemm_stream_kernel(StreamParams p) {
+// NS = sub-tiles per pass.
+template <int MODE, bool kFused, int NS>
+__global__ __launch_bounds__(kThreads, NS == 1 ? 3 : 2) void gemm_stream_kernel(StreamParams p) {
   __shared__ __align__(16) char lds[kWaves * kWaveLds];
   __shared__ __align__(16) char a_lds[kFused ? kSub * (kFusedMaxK + kFusedRowPad) : 16];
   __shared__ float s_lds[kSub];
@@ -332,11 +338,10 @@ __global__ __launch_bounds__(kThreads, 3) void gemm_stream_kernel(StreamParams p
   // Valid rows are a prefix of the block (at least one, the block is in use): the first pass counts
   // them to know how many sub-tiles there are.
   char* wave_lds = lds + (threadIdx.x / kWave) * kWaveLds;
-  const int nvalid =
-      stream_pass<MODE, kGroup, kFused>(p, blk, e, 0, first_pair, npairs, wave_lds, true, a_lds, s_lds);
+  const int nvalid = stream_pass<MODE, NS, kFused>(p, blk, e, 0, first_pair, npairs, wave_lds, true, a_lds, s_lds);
   const int nsub = (nvalid + kSub - 1) / kSub;
-  for (int sub0 = kGroup; sub0 < nsub; sub0 += kGroup)
-    stream_pass<MODE, kGroup, kFused>(p, blk, e, sub0, first_pair, npairs, wave_lds, false, a_lds, s_lds);
+  for (int sub0 = NS; sub0 < nsub; sub0 += NS)
+    stream_pass<MODE, NS, kFused>(p, blk, e, sub0, first_pair, npairs, wave_lds, false, a_lds, s_lds);
 }
 
 template <int MODE, bool kFused = false>
@@ -368,7 +373,10 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   if (blocks == 0 || waves == 0) return hipSuccess;
   if (blocks > 65535) return hipErrorInvalidValue;
   const dim3 grid((unsigned)((waves + kWaves - 1) / kWaves), (unsigned)blocks);
-  hipLaunchKernelGGL((gemm_stream_kernel<MODE, kFused>), grid, dim3(kThreads), 0, stream, p);
+  if (!kFused && a.num_pairs > (int64_t)kPairRowsPerExpert * a.num_experts)
+    hipLaunchKernelGGL((gemm_stream_kernel<MODE, kFused, kFused ? 1 : 2>), grid, dim3(kThreads), 0, stream, p);
+  else
+    hipLaunchKernelGGL((gemm_stream_kernel<MODE, kFused, 1>), grid, dim3(kThreads), 0, stream, p);
   return hipGetLastError();
 }
 
