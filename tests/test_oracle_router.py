@@ -127,3 +127,16 @@ def test_routed_experts_record_reference_payloads(oracle):
     assert wide["dtype"] == "uint16" and wide["start"] == 4
     assert np.frombuffer(base64.b64decode(wide["data"]), dtype=np.uint16).tolist() == [1, 511]
     assert oracle.serialize_routed_experts(None) is None
+
+
+def test_golden_vectors(oracle, golden):
+    g = golden["router_ties"]
+    _, ids = oracle.route_topk(torch.tensor([g["logits"]]), 5, "topk_softmax", False)
+    assert ids.tolist() == [g["top5_ids"]]
+    _, ids = oracle.route_topk(torch.tensor([g["grouped_logits"]]), 2, "topk_softmax", False,
+                               num_groups=g["grouped_num_groups"], topk_groups=g["grouped_topk_groups"])
+    assert ids.tolist() == [g["grouped_top2_ids"]]
+    r = golden["routed_experts_payloads"]
+    enc = oracle.serialize_routed_experts(np.array(r["array"], dtype=np.int64))
+    assert enc["data"] == r["array_base64"] and list(base64.b64decode(enc["data"])) == r["array_bytes"]
+    assert oracle.serialize_routed_experts(np.array(r["compact_ids"])) == r["compact"]

@@ -92,3 +92,13 @@ def test_quantised_layer_tracks_the_bf16_layer(oracle):
     want = oracle.dequant_fp32_moe(x, torch.cat([gate, up], 1).float(), down.float(), tw, ids, ones13, ones2).float()
     rel = (got - want).norm() / want.norm()
     assert rel < 0.05, rel
+
+
+def test_golden_tie_vector(oracle, golden):
+    g = golden["weight_quant_ties"]
+    q, s = oracle.quantize_weights_per_channel(torch.tensor([g["w"]], dtype=torch.bfloat16))
+    assert q.tolist() == [g["q_half_even"]] and s.tolist() == [g["scale"]]
+    qd, sd = oracle.scaled_int8_quant(torch.tensor([g["w"]], dtype=torch.bfloat16))
+    assert qd.tolist() == [g["q_half_even"]] and sd.tolist() == [[g["scale"]]]
+    _, z = oracle.quantize_weights_per_channel(torch.zeros(1, 8, dtype=torch.bfloat16))
+    assert z.item() == np.float32(g["zero_row_scale"])
