@@ -129,6 +129,41 @@ def test_python_wrappers_refuse_cpu_tensors_and_unsupported_modes(pra):
         pra.moe_align_block_size(ids, 64, 2, expert_map=torch.zeros(2))
 
 
+def test_widened_wrappers_refuse_cpu_tensors_and_unsupported_modes(pra):
+    x = torch.zeros((4, 128), dtype=torch.bfloat16)
+    logits = torch.zeros((4, 8))
+    w = torch.zeros((8, 128), dtype=torch.int8)
+    ws = torch.ones(8)
+    for call in (
+        lambda: pra.route_topk(logits, 2),
+        lambda: pra.fused_topk(x, logits, 2, True),
+        lambda: pra.grouped_topk(x, logits, 2, True, 2, 1),
+        lambda: pra.quantize_weights_per_channel(x),
+        lambda: pra.quantize_expert_weights(x.view(1, 4, 128), x.view(1, 4, 128), x.view(1, 128, 4)),
+        lambda: pra.scaled_int8_quant(x),
+        lambda: pra.apply_int8_linear(x, w, ws),
+        lambda: pra.w8a8_mlp(x, w, ws, w, ws),
+        lambda: pra.moe_sum(torch.zeros(4, 2, 128, dtype=torch.bfloat16), x),
+    ):
+        with pytest.raises(ValueError, match="GPU tensor"):
+            call()
+    with pytest.raises(ValueError, match="tokens mismatch"):
+        pra.fused_topk(x[:2], logits, 2, True)
+    with pytest.raises(ValueError, match="Unsupported scoring"):
+        pra.grouped_topk(x, logits, 2, True, 2, 1, "tanh")
+    with pytest.raises(NotImplementedError):
+        pra.scaled_int8_quant(x, scale=torch.ones(1))
+    with pytest.raises(NotImplementedError):
+        pra.apply_int8_linear(x, w, ws, input_scale=torch.ones(1))
+    with pytest.raises(NotImplementedError):
+        pra.fused_moe(x, w, w, logits, 2, True, custom_routing_function=lambda *a: None)
+    with pytest.raises(ValueError, match="record must be"):
+        pra.routed_experts_payload(torch.zeros(4, 2, dtype=torch.uint8))
+    # the wire form of a record needs no GPU: field for field the reference's dictionary
+    rec = torch.tensor([[[1, 2, 3]]], dtype=torch.uint8)
+    assert pra.routed_experts_payload(rec) == {"data": "AQID", "shape": [1, 1, 3], "start": 0, "dtype": "uint8"}
+
+
 def test_fused_experts_signature_is_vllms(pra):
     import inspect
 
