@@ -336,7 +336,7 @@ __device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, in
         const int32_t t = __shfl(tok[tj], row);
         const int n = n0 + chunk * 8;
         if (t >= 0 && n < p.N)
-          *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.out) + (int64_t)t * p.N + n) = v;
+          __builtin_nontemporal_store(v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w}, reinterpret_cast<v4i*>(static_cast<uint16_t*>(p.out) + (int64_t)t * p.N + n));
       }
     }
   } else {
@@ -371,7 +371,7 @@ __device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, in
       const int32_t t = __shfl(tok[r >> 2], row & 31);
       const int n = n0 + chunk * 8;
       if (t >= 0 && n < inter)
-        *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.out) + (int64_t)t * inter + n) = v;
+        __builtin_nontemporal_store(v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w}, reinterpret_cast<v4i*>(static_cast<uint16_t*>(p.out) + (int64_t)t * inter + n));
     }
   }
 }
