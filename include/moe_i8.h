@@ -190,6 +190,9 @@ int64_t moe_i8_workspace_bytes(int64_t m, int top_k, int num_experts, int hidden
  * (model_executor/layers/fused_moe/fused_moe.py): quant, align, gate_up GEMM +
  * SiLU*mul, quant, down GEMM * routed weight, sum — all on `stream`, no host
  * synchronisation.  hidden bf16 [M, H]; out bf16 [M, H] (may alias hidden).
+ * Every topk_id must lie in [0, num_experts): a pair with another id is skipped by the alignment and
+ * the GEMMs, so its row of the intermediate buffer is never written and the combine would add
+ * whatever the workspace holds there (expert-parallel maps are not part of this path).
  */
 int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
                          const float* topk_weights, const int32_t* topk_ids,

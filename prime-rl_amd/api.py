@@ -674,6 +674,8 @@ def fused_experts(
     per-token dynamic quantisation upstream recomputes them too.  The three keyword-only
     arguments are extensions: the moe_align block size (64, as the baseline pins it), the GEMM
     kernel family and an optional caller-owned workspace of ``workspace_bytes(...)`` bytes.
+    ``topk_ids`` must lie in ``[0, E)``: there is no expert map on this path, and a pair routed
+    nowhere would leave its row of the intermediate buffer unwritten.
     """
     if not use_int8_w8a8:
         raise NotImplementedError("this library implements only the use_int8_w8a8=True path")
