@@ -189,3 +189,23 @@ def test_missing_library_fails_loudly(pra, monkeypatch, tmp_path):
     monkeypatch.setattr(pra._abi, "LIB_PATH", tmp_path / "libmoe_i8.so")
     with pytest.raises(ImportError, match="no CPU or PyTorch fallback"):
         pra._abi.load()
+
+
+def test_header_is_plain_c_and_a_c_client_links(pra, tmp_path):
+    """include/moe_i8.h compiles as C99 and a C program linked against the library gets the documented
+    sizes and argument errors (no GPU needed for any of these calls)."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    root = ROOT
+    lib = pra._abi.LIB_PATH
+    exe = tmp_path / "abi_check"
+    cmd = [gcc, "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", str(root / "include"),
+           str(root / "tests" / "c" / "abi_check.c"), "-o", str(exe), str(lib), f"-Wl,-rpath,{lib.parent}",
+           "-Wl,-rpath,/opt/rocm/lib"]
+    subprocess.run(cmd, check=True, capture_output=True, text=True)
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0 and run.stdout.strip() == "ok", run.stdout + run.stderr
