@@ -307,6 +307,27 @@ int moe_i8_gemm_gate_up_silu(const int8_t* x_q, const float* a_scale, const int8
   g.block_size = block_size;
   g.sorted_cap = sorted_cap;
   g.out = act_out;
+  g.max_rows_per_expert = (num_pairs + top_k - 1) / top_k;  // an expert sees a token at most once
+  return run_gemm(g, variant, static_cast<hipStream_t>(stream));
+}
+
+// The down GEMM behind the entry point; `max_rows` bounds the rows any one expert can hold (0: unknown).
+static int gemm_down_impl(const int8_t* h_q, const float* a_scale, const int8_t* w2, const float* w2_scale,
+                          const float* topk_weights, const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                          const int32_t* num_tokens_post_padded, int64_t num_pairs, int num_experts, int hidden,
+                          int inter, int block_size, int64_t sorted_cap, void* out, int variant, int64_t max_rows,
+                          void* stream) {
+  if (num_pairs == 0) return MOE_I8_OK;
+  if (int rc = check_gemm_common(h_q, w2, sorted_token_ids, expert_ids, num_tokens_post_padded, out,
+                                 num_pairs, num_experts, hidden, inter, block_size, sorted_cap,
+                                 variant))
+    return rc;
+  if (!a_scale || !w2_scale) return fail(MOE_I8_EINVAL, "null scale pointer");
+  if (!aligned16(w2_scale)) return fail(MOE_I8_EINVAL, "w2_scale must be 16-byte aligned");
+  moe_i8::GemmArgs g = down_args(h_q, a_scale, w2, w2_scale, topk_weights, sorted_token_ids, expert_ids,
+                                 num_tokens_post_padded, num_pairs, num_experts, hidden, inter, block_size,
+                                 sorted_cap, out);
+  g.max_rows_per_expert = max_rows;
   return run_gemm(g, variant, static_cast<hipStream_t>(stream));
 }
 
@@ -316,17 +337,9 @@ int moe_i8_gemm_down(const int8_t* h_q, const float* a_scale, const int8_t* w2,
                      const int32_t* num_tokens_post_padded, int64_t num_pairs, int num_experts,
                      int hidden, int inter, int block_size, int64_t sorted_cap, void* out,
                      int variant, void* stream) {
-  if (num_pairs == 0) return MOE_I8_OK;
-  if (int rc = check_gemm_common(h_q, w2, sorted_token_ids, expert_ids, num_tokens_post_padded, out,
-                                 num_pairs, num_experts, hidden, inter, block_size, sorted_cap,
-                                 variant))
-    return rc;
-  if (!a_scale || !w2_scale) return fail(MOE_I8_EINVAL, "null scale pointer");
-  if (!aligned16(w2_scale)) return fail(MOE_I8_EINVAL, "w2_scale must be 16-byte aligned");
-  return run_gemm(down_args(h_q, a_scale, w2, w2_scale, topk_weights, sorted_token_ids, expert_ids,
-                            num_tokens_post_padded, num_pairs, num_experts, hidden, inter, block_size, sorted_cap,
-                            out),
-                  variant, static_cast<hipStream_t>(stream));
+  return gemm_down_impl(h_q, a_scale, w2, w2_scale, topk_weights, sorted_token_ids, expert_ids,
+                        num_tokens_post_padded, num_pairs, num_experts, hidden, inter, block_size, sorted_cap, out,
+                        variant, 0, stream);
 }
 
 int moe_i8_gemm_down_bf16(const void* act, const int8_t* w2, const float* w2_scale, const float* topk_weights,
@@ -512,8 +525,8 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
   } else {
     if (int rc = moe_i8_quant_rows(act, MOE_I8_DTYPE_BF16, p, inter, inter, nullptr, 1, p, act_q, a2, stream))
       return rc;
-    if (int rc = moe_i8_gemm_down(act_q, a2, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
-                                  hidden_size, inter, block_size, c.cap, down, variant, stream))
+    if (int rc = gemm_down_impl(act_q, a2, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
+                                hidden_size, inter, block_size, c.cap, down, variant, m, stream))
       return rc;
   }
   return moe_i8_sum(down, out, m, top_k, hidden_size, stream);

@@ -187,6 +187,7 @@ struct GemmArgs {
   int block_size;
   int64_t sorted_cap;
   void* out;  // bf16 [P, I] | bf16 [P, H] | int32 [P, N]
+  int64_t max_rows_per_expert = 0;  // upper bound if the caller knows one (the token count), else 0
 };
 hipError_t launch_gemm_stream(const GemmArgs& a, hipStream_t stream);
 bool gemm_stream_fuses_quant(int k);  // the down GEMM can quantise bf16 activations of this length itself

@@ -335,9 +335,20 @@ __global__ __launch_bounds__(kThreads, NS == 1 ? 3 : 2) void gemm_stream_kernel(
   const int left = total_pairs - first_pair;
   const int npairs = left < 0 ? 0 : left < p.pairs_per_wave ? left : p.pairs_per_wave;
 
-  // Valid rows are a prefix of the block (at least one, the block is in use): the first pass counts
-  // them to know how many sub-tiles there are.
   char* wave_lds = lds + (threadIdx.x / kWave) * kWaveLds;
+  if (gridDim.z > 1) {
+    // The passes of a block are spread over grid.z workgroups (they run side by side instead of one
+    // after the other, which matters when a few experts hold most rows).  Valid rows are a prefix
+    // of the block: a pass whose first row is padding has nothing to do.
+    const int sub0 = blockIdx.z * NS;
+    if (sub0 * kSub >= p.B) return;
+    const int32_t t = p.sorted_ids[(int64_t)blk * p.B + sub0 * kSub];
+    if (t < 0 || t >= p.P) return;
+    stream_pass<MODE, NS, kFused>(p, blk, e, sub0, first_pair, npairs, wave_lds, false, a_lds, s_lds);
+    return;
+  }
+  // One workgroup walks all passes; the first one counts the valid rows (a prefix of the block, at
+  // least one: the block is in use) to know how many sub-tiles there are.
   const int nvalid = stream_pass<MODE, NS, kFused>(p, blk, e, 0, first_pair, npairs, wave_lds, true, a_lds, s_lds);
   const int nsub = (nvalid + kSub - 1) / kSub;
   for (int sub0 = NS; sub0 < nsub; sub0 += NS)
@@ -372,8 +383,16 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   const int64_t blocks = (a.sorted_cap + a.block_size - 1) / a.block_size;
   if (blocks == 0 || waves == 0) return hipSuccess;
   if (blocks > 65535) return hipErrorInvalidValue;
-  const dim3 grid((unsigned)((waves + kWaves - 1) / kWaves), (unsigned)blocks);
-  if (!kFused && a.num_pairs > (int64_t)kPairRowsPerExpert * a.num_experts)
+  const bool two = !kFused && a.num_pairs > (int64_t)kPairRowsPerExpert * a.num_experts;
+  // Passes per block that can be needed: no expert holds more rows than there are tokens (or pairs,
+  // when the caller did not say).  One workgroup per pass once there can be more than one.
+  const int ns = two ? 2 : 1;
+  const int64_t most_rows = a.max_rows_per_expert > 0 && a.max_rows_per_expert < a.num_pairs ? a.max_rows_per_expert
+                                                                                             : a.num_pairs;
+  const int64_t rows = most_rows < a.block_size ? most_rows : a.block_size;
+  const int passes = kFused ? 1 : (int)((rows + kSub * ns - 1) / (kSub * ns));
+  const dim3 grid((unsigned)((waves + kWaves - 1) / kWaves), (unsigned)blocks, (unsigned)(passes > 1 ? passes : 1));
+  if (two)
     hipLaunchKernelGGL((gemm_stream_kernel<MODE, kFused, kFused ? 1 : 2>), grid, dim3(kThreads), 0, stream, p);
   else
     hipLaunchKernelGGL((gemm_stream_kernel<MODE, kFused, 1>), grid, dim3(kThreads), 0, stream, p);
