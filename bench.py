@@ -230,6 +230,32 @@ def time_router(pkg, torch, shape, M: int, steps: int, warmup: int) -> dict:
     return {"M": M, "us": t * 1e6, "bytes": nbytes, "hbm_gbps": nbytes / t / 1e9}
 
 
+def time_mfma_ceiling(pkg, torch) -> dict:
+    """What the device sustains on a register-only int8 MFMA loop (no memory traffic at all) with constant
+    and with pseudo-random operand bits: the board's power limit lowers the clock as the operand bits
+    toggle, so the second figure, not the published peak, is the ceiling of any int8 GEMM on real data
+    here.  One launch of a few milliseconds on one workgroup per compute unit, best of four."""
+    lib, abi = pkg._abi.load(), pkg._abi
+    wgs = torch.cuda.get_device_properties(0).multi_processor_count
+    iters = 20000
+    sink = torch.empty(wgs * 512, dtype=torch.int32, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    ops = lib.moe_i8_probe_mfma_ops(wgs, iters)
+    res = {"unit": "TFLOP/s", "note": "int8 TOP/s, v_mfma_i32_32x32x32_i8 from registers on every compute unit"}
+    for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
+        best = float("inf")
+        for _ in range(4):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            abi.check(lib.moe_i8_probe_mfma(rnd, wgs, iters, sink.data_ptr(), sink.numel() * 4, stream))
+            b.record()
+            torch.cuda.synchronize()
+            best = min(best, a.elapsed_time(b) * 1e-3)
+        res[name] = ops / best / 1e12
+        res[name + "_frac_of_peak"] = ops / best / PEAK_INT8_OPS
+    return res
+
+
 def time_dense_mlp(pkg, torch, M: int, H: int, I: int, steps: int, warmup: int) -> dict:
     """The shared-expert / dense W8A8 gated MLP on the same GEMM kernels with one group."""
     g = torch.Generator(device="cuda:0").manual_seed(3)
@@ -373,6 +399,7 @@ def main() -> int:
                             for M in (args.m, 8 * args.m)]
         out["weight_requant"] = time_weight_requant(pkg, torch, pkg.inputs.SHAPES[args.shape],
                                                     max(args.steps // 2, 1), max(args.warmup // 2, 1))
+        out["mfma_ceiling"] = time_mfma_ceiling(pkg, torch)
     if not args.no_cpu:
         oracle = importlib.import_module("oracle.moe_i8_oracle")
         out["cpu_baseline"] = cpu_baseline(oracle, torch, base_headline, args.cpu_sample)

@@ -190,6 +190,10 @@ struct GemmArgs {
   int64_t max_rows_per_expert = 0;  // upper bound if the caller knows one (the token count), else 0
 };
 hipError_t launch_gemm_stream(const GemmArgs& a, hipStream_t stream);
+// register-only int8 MFMA loop (measurement aid): sink holds mfma_probe_sink_bytes(workgroups)
+int64_t mfma_probe_sink_bytes(int workgroups);
+double mfma_probe_ops(int workgroups, int iters);
+hipError_t launch_mfma_probe(bool random_operands, int workgroups, int iters, int32_t* sink, hipStream_t stream);
 bool gemm_stream_fuses_quant(int k);  // the down GEMM can quantise bf16 activations of this length itself
 hipError_t launch_gemm_tile(const GemmArgs& a, hipStream_t stream);
 bool gemm_tile_supports(const GemmArgs& a);

@@ -164,3 +164,35 @@ def test_decode_mix_sequence_reuses_workspace(pra, oracle):
                                     sub["w1_scale"], sub["w2_scale"], 64)
         err = rel_err(out[sel.to(DEV)], want)
         assert err < TOL, (step, M, err)
+
+
+@pytest.mark.parametrize("E,k,H,I,M,B", [
+    (128, 8, 2048, 768, 1, 64), (128, 8, 2048, 768, 16, 64), (128, 8, 2048, 768, 48, 64),
+    (8, 2, 256, 128, 12, 16), (16, 3, 512, 256, 16, 64), (24, 4, 320, 1024, 18, 32), (64, 6, 1024, 512, 32, 64),
+    (4, 1, 64, 64, 12, 16), (2, 2, 2048, 64, 3, 128), (8, 8, 192, 192, 3, 64),
+])
+def test_small_batch_layer_equals_the_chain_of_its_stages(pra, E, k, H, I, M, B):
+    """With a handful of rows per expert the layer merges launches (moe_align with the first
+    quantisation, the second quantisation with the down GEMM).  The result must equal, bit for bit,
+    the six stand-alone stages called one after the other — on skewed routing too, where one block
+    holds several 16-row passes — and must not depend on what the workspace held."""
+    im = inputs_mod()
+    for routing in ("softmax", "zipf"):
+        shape = im.LayerShape("s", E=E, k=k, H=H, I=I, routing=routing)
+        inp = im.make_inputs(shape, M, seed=M + E).to(DEV)
+        P = M * k
+        x_q, a1 = pra.per_token_quant_int8(inp.hidden_states)
+        s, e, npp = pra.moe_align_block_size(inp.topk_ids, B, E)
+        act = pra.gemm_gate_up_silu(x_q, a1, inp.w1, inp.w1_scale, s, e, npp, k, B, P, "stream")
+        h_q, a2 = pra.per_token_quant_int8(act)
+        down = pra.gemm_down(h_q, a2, inp.w2, inp.w2_scale, inp.topk_weights, s, e, npp, B, "stream")
+        want = torch.empty(M, H, dtype=torch.bfloat16, device=DEV)
+        pra.moe_sum(down.view(M, k, H), want)
+        ws = torch.empty((pra.workspace_bytes(M, k, E, H, I, B),), dtype=torch.uint8, device=DEV)
+        for fill in (0, 0xFF, 0x5A):
+            ws.fill_(fill)
+            out = pra.fused_experts(*inp.fused_experts_args(), **inp.fused_experts_kwargs(), block_size_m=B,
+                                    workspace=ws, gemm_variant="stream")
+            torch.cuda.synchronize()
+            same = bool(torch.equal(out, want))
+            assert same, (routing, fill, int((out != want).sum()))
