@@ -16,7 +16,7 @@ LIB_PATH = PKG_DIR / "libmoe_i8.so"
 OK = 0
 EINVAL, EWORKSPACE, ELAUNCH, EUNSUPPORTED = -1, -2, -3, -4
 DTYPE_BF16 = 0
-GEMM_AUTO, GEMM_STREAM, GEMM_TILE = 0, 1, 2
+GEMM_AUTO, GEMM_STREAM, GEMM_TILE, GEMM_NARROW = 0, 1, 2, 3
 SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_TOPK_SOFTMAX = 0, 1, 2
 MAX_EXPERTS = 1024
 

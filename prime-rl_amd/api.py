@@ -41,7 +41,7 @@ __all__ = [
 ]
 
 DEFAULT_BLOCK_SIZE_M = 64
-_VARIANTS = {"auto": _abi.GEMM_AUTO, "stream": _abi.GEMM_STREAM, "tile": _abi.GEMM_TILE}
+_VARIANTS = {"auto": _abi.GEMM_AUTO, "stream": _abi.GEMM_STREAM, "tile": _abi.GEMM_TILE, "narrow": _abi.GEMM_NARROW}
 _workspaces: dict[tuple[int, int], torch.Tensor] = {}
 
 

@@ -11,7 +11,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libmoe_i8.so"
-SOURCES = ["align.hip", "quant.hip", "sum.hip", "router.hip", "gemm_stream.hip", "gemm_tile.hip", "probe.hip", "api.hip"]
+SOURCES = ["align.hip", "quant.hip", "sum.hip", "router.hip", "gemm_stream.hip", "gemm_tile.hip", "gemm_narrow.hip", "probe.hip", "api.hip"]
 
 # packed-fp32 VALU ops are switched off for all device code (hipcc's host pass warns that it does
 # not know the feature; that is harmless).

@@ -43,31 +43,48 @@ int check_gemm_common(const void* a_q, const void* w, const int32_t* sorted, con
   if (k < 64 || k % 64) return fail(MOE_I8_EINVAL, "reduction length (%d) must be a positive multiple of 64", k);
   if (sorted_cap < moe_i8_sorted_capacity(num_pairs, num_experts, block_size))
     return fail(MOE_I8_EWORKSPACE, "sorted_token_ids capacity %lld too small", (long long)sorted_cap);
-  if (variant != MOE_I8_GEMM_AUTO && variant != MOE_I8_GEMM_STREAM && variant != MOE_I8_GEMM_TILE)
+  if (variant != MOE_I8_GEMM_AUTO && variant != MOE_I8_GEMM_STREAM && variant != MOE_I8_GEMM_TILE &&
+      variant != MOE_I8_GEMM_NARROW)
     return fail(MOE_I8_EINVAL, "unknown GEMM variant %d", variant);
   return MOE_I8_OK;
 }
 
-// Which family a launch goes to; -1 with the error set if the tile family was demanded for a shape
-// it does not handle.
-int picks_tile(const moe_i8::GemmArgs& g, int variant) {
+constexpr int kStreamRowsPerExpert = 12;
+constexpr int kNarrowRowsPerExpert = 56;
+
+// Which family a launch goes to (one of the MOE_I8_GEMM_* constants, never AUTO); -1 with the error
+// set if a family was demanded for a shape it does not handle.
+int picks_family(const moe_i8::GemmArgs& g, int variant) {
   if (variant == MOE_I8_GEMM_TILE) {
     if (!moe_i8::gemm_tile_supports(g))
       return fail(MOE_I8_EUNSUPPORTED, "tile GEMM does not support this shape"), -1;
-    return 1;
+    return MOE_I8_GEMM_TILE;
   }
-  if (variant == MOE_I8_GEMM_STREAM) return 0;
-  // Measured crossover on the Qwen3-30B-A3B shape: the streaming family wins while a block holds
-  // one or two 16-row sub-tiles (up to about 24 routed rows per expert), the LDS-tiled family beyond.
-  return moe_i8::gemm_tile_supports(g) && g.num_pairs > (int64_t)24 * g.num_experts;
+  if (variant == MOE_I8_GEMM_NARROW) {
+    if (!moe_i8::gemm_narrow_supports(g))
+      return fail(MOE_I8_EUNSUPPORTED, "narrow-tile GEMM does not support this shape"), -1;
+    return MOE_I8_GEMM_NARROW;
+  }
+  if (variant == MOE_I8_GEMM_STREAM) return MOE_I8_GEMM_STREAM;
+  // Measured crossovers on the Qwen3-30B-A3B shape, in routed rows per expert: the streaming family
+  // wins while a block mostly holds one 16-row sub-tile (up to about 12), the narrow tiles while
+  // most experts hold a single 64-row block (up to about 56), the wide LDS tiles beyond.
+  const int64_t rows_x_experts = g.num_pairs;
+  if (rows_x_experts <= (int64_t)kStreamRowsPerExpert * g.num_experts) return MOE_I8_GEMM_STREAM;
+  if (rows_x_experts <= (int64_t)kNarrowRowsPerExpert * g.num_experts && moe_i8::gemm_narrow_supports(g))
+    return MOE_I8_GEMM_NARROW;
+  if (moe_i8::gemm_tile_supports(g)) return MOE_I8_GEMM_TILE;
+  return moe_i8::gemm_narrow_supports(g) ? MOE_I8_GEMM_NARROW : MOE_I8_GEMM_STREAM;
 }
 
 int run_gemm(const moe_i8::GemmArgs& g, int variant, hipStream_t stream) {
   if (g.num_pairs == 0) return MOE_I8_OK;
-  const int tile = picks_tile(g, variant);
-  if (tile < 0) return MOE_I8_EUNSUPPORTED;
-  return check_launch(tile ? moe_i8::launch_gemm_tile(g, stream) : moe_i8::launch_gemm_stream(g, stream),
-                      tile ? "gemm_tile" : "gemm_stream");
+  switch (picks_family(g, variant)) {
+    case MOE_I8_GEMM_TILE: return check_launch(moe_i8::launch_gemm_tile(g, stream), "gemm_tile");
+    case MOE_I8_GEMM_NARROW: return check_launch(moe_i8::launch_gemm_narrow(g, stream), "gemm_narrow");
+    case MOE_I8_GEMM_STREAM: return check_launch(moe_i8::launch_gemm_stream(g, stream), "gemm_stream");
+    default: return MOE_I8_EUNSUPPORTED;
+  }
 }
 
 moe_i8::GemmArgs down_args(const int8_t* h_q, const float* a_scale, const int8_t* w2, const float* w2_scale,
@@ -516,9 +533,9 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
   // per expert on (measured) the separate launch is the cheaper one again.
   const moe_i8::GemmArgs dg = down_args(act_q, a2, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
                                         hidden_size, inter, block_size, c.cap, down);
-  const int down_tile = picks_tile(dg, variant);
-  if (down_tile < 0) return MOE_I8_EUNSUPPORTED;
-  if (!down_tile && moe_i8::gemm_stream_fuses_quant(inter) && p <= (int64_t)3 * num_experts) {
+  const int down_family = picks_family(dg, variant);
+  if (down_family < 0) return MOE_I8_EUNSUPPORTED;
+  if (down_family == MOE_I8_GEMM_STREAM && moe_i8::gemm_stream_fuses_quant(inter) && p <= (int64_t)3 * num_experts) {
     if (int rc = moe_i8_gemm_down_bf16(act, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
                                        hidden_size, inter, block_size, c.cap, down, stream))
       return rc;

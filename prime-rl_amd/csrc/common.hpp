@@ -197,6 +197,8 @@ hipError_t launch_mfma_probe(bool random_operands, int workgroups, int iters, in
 bool gemm_stream_fuses_quant(int k);  // the down GEMM can quantise bf16 activations of this length itself
 hipError_t launch_gemm_tile(const GemmArgs& a, hipStream_t stream);
 bool gemm_tile_supports(const GemmArgs& a);
+hipError_t launch_gemm_narrow(const GemmArgs& a, hipStream_t stream);
+bool gemm_narrow_supports(const GemmArgs& a);
 
 hipError_t launch_moe_sum(const uint16_t* in, uint16_t* out, int64_t m, int top_k, int hidden,
                           hipStream_t stream);

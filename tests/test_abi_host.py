@@ -88,6 +88,9 @@ def test_c_abi_rejects_bad_arguments_without_launching(pra):
     assert call(H=96) == abi.EINVAL
     assert call(I=24) == abi.EINVAL
     assert call(variant=9) == abi.EINVAL
+    # a family demanded for a shape it does not handle: refused before anything is launched
+    assert call(H=128, variant=abi.GEMM_TILE) == abi.EUNSUPPORTED and "tile" in err()
+    assert call(H=384, variant=abi.GEMM_NARROW) == abi.EUNSUPPORTED and "narrow" in err()
     assert call(x=None) == abi.EINVAL
     assert lib.moe_i8_gemm_down(p, p, p, p, p, p, p, p, 8, 4, 128, 100, 64, 260, p, 0, None) == abi.EINVAL
     assert lib.moe_i8_gemm_acc_i32(p, p, p, p, p, 8, 0, 4, 128, 128, 64, 260, p, 0, None) == abi.EINVAL

@@ -47,22 +47,29 @@ def test_random_shape(pra, oracle, case):
     x_q, h_q = st["x_q"].to(DEV), st["h_q"].to(DEV)
     a2 = st["a2_scale"].to(DEV)
     ran = 0
-    for variant in ("stream", "tile"):
+    def attempt(fn):
         try:
-            acc1 = pra.gemm_acc_i32(x_q, d.w1, s, e, npp, k, B, P, variant)
-            acc2 = pra.gemm_acc_i32(h_q, d.w2, s, e, npp, 1, B, P, variant)
-            down = pra.gemm_down(h_q, a2, d.w2, d.w2_scale, d.topk_weights, s, e, npp, B, variant)
+            return fn()
         except pra._abi.MoeI8Error as exc:
             if exc.code == pra._abi.EUNSUPPORTED:
-                continue
+                return None
             raise
-        ran += 1
-        assert torch.equal(acc1.cpu(), st["acc1"]), (variant, int((acc1.cpu() != st["acc1"]).sum()))
-        assert torch.equal(acc2.cpu(), st["acc2"]), (variant, int((acc2.cpu() != st["acc2"]).sum()))
-        want = st["cache3"].reshape(P, H)
-        assert torch.equal(down.cpu(), want), (variant, int((down.cpu() != want).sum()))
+
+    want = st["cache3"].reshape(P, H)
+    for variant in ("stream", "tile", "narrow"):
+        # a family may support one of the two GEMM shapes of a layer and not the other
+        acc1 = attempt(lambda: pra.gemm_acc_i32(x_q, d.w1, s, e, npp, k, B, P, variant))
+        acc2 = attempt(lambda: pra.gemm_acc_i32(h_q, d.w2, s, e, npp, 1, B, P, variant))
+        down = attempt(lambda: pra.gemm_down(h_q, a2, d.w2, d.w2_scale, d.topk_weights, s, e, npp, B, variant))
+        if acc1 is not None:
+            ran += 1
+            assert torch.equal(acc1.cpu(), st["acc1"]), (variant, int((acc1.cpu() != st["acc1"]).sum()))
+        if acc2 is not None:
+            assert torch.equal(acc2.cpu(), st["acc2"]), (variant, int((acc2.cpu() != st["acc2"]).sum()))
+        if down is not None:
+            assert torch.equal(down.cpu(), want), (variant, int((down.cpu() != want).sum()))
     assert ran >= 1
-    for variant in ("auto", "tile"):
+    for variant in ("auto", "tile", "narrow"):
         try:
             out = pra.fused_experts(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, use_int8_w8a8=True,
                                     per_channel_quant=True, w1_scale=d.w1_scale, w2_scale=d.w2_scale,
