@@ -41,6 +41,7 @@ constexpr int kTokOffset = kCh * kBK;
 constexpr int kStageBytes = (kCh + kTok) * kBK;  // 24 KB
 constexpr int kStageLoads = 6;                   // 1 KB loads per wavefront and step: 4 weight + 2 token
 constexpr int kXcds = 8;
+constexpr int kFirstGroup = 2;                   // the last loads of the start-up: token rows of step 1
 constexpr int kMinSteps = 4;  // the look-ahead of the next tile's inputs needs this many steps per tile
 
 // Inputs of one tile's epilogue (and of the loads of its token rows), filled by 4-byte global -> LDS
@@ -103,14 +104,16 @@ __device__ __forceinline__ void load_to_lds_4(const void* base, uint32_t offset,
                : "memory", "m0");
 }
 
-// One int from a wave-uniform address through the scalar (read-only) path.  After the inline
-// assembly above the compiler no longer proves that global memory is unchanged and would fetch such
-// a value with a vector load, whose wait would drain the ring; this one only waits for itself.
-// Only for data written before the launch (the scalar cache does not see this kernel's stores).
-__device__ __forceinline__ int32_t scalar_load(const int32_t* p) {
-  int32_t v;
-  asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(uniform_address(p)) : "memory");
-  return v;
+// Two ints from wave-uniform addresses through the scalar (read-only) path, one wait for both.
+// After the inline assembly above the compiler no longer proves that global memory is unchanged and
+// would fetch such values with vector loads, whose wait would drain the ring; this only waits for
+// itself.  Only for data written before the launch (the scalar cache does not see this kernel's
+// stores).
+__device__ __forceinline__ void scalar_load2(const int32_t* pa, const int32_t* pb, int32_t& a, int32_t& b) {
+  asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+               : "=&s"(a), "=&s"(b)
+               : "s"(uniform_address(pa)), "s"(uniform_address(pb))
+               : "memory");
 }
 
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
@@ -138,11 +141,13 @@ constexpr int aux_loads() {
 }
 
 // Waits until at most the `n` most recent vector-memory operations of this wavefront are pending;
-// n is the size of the group issued last, one of three values.
+// n is the size of the group issued last, one of four values.
 template <int MODE>
 __device__ __forceinline__ void wait_all_but(int n) {
   if (n == kStageLoads)
     wait_vmcnt<kStageLoads>();
+  else if (n == kFirstGroup)
+    wait_vmcnt<kFirstGroup>();
   else if (n == kStageLoads + 1)
     wait_vmcnt<kStageLoads + 1>();
   else
@@ -184,9 +189,9 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_narrow_kernel(NarrowParams p
       const int task = xcd * per_xcd + it;
       const int tile = task / p.ntiles;
       const int blk = tile / sub_per_block;
-      const int e = scalar_load(p.expert_ids + blk);
       const int64_t slot0 = (int64_t)blk * p.B + (int64_t)(tile % sub_per_block) * kTok;
-      const int32_t first = scalar_load(p.sorted_ids + slot0);
+      int32_t e, first;
+      scalar_load2(p.expert_ids + blk, p.sorted_ids + slot0, e, first);
       if (e >= 0 && e < p.E && first >= 0 && first < p.P) {
         tk.e = e;
         tk.ct = task - tile * p.ntiles;
@@ -202,7 +207,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_narrow_kernel(NarrowParams p
   // ---- global -> LDS loads ----
   // Lane fills LDS slot (lane & 7) of row base + 8 * i + (lane >> 3): it fetches the logical chunk
   // (lane & 7) ^ swizzle(row) of that row, and swizzle(row) = (lane >> 3) ^ (i & 1).
-  auto setup_loads = [&](const Task& tk, const TileAux& ax, TaskLoads& ld) {
+  auto setup_weight_loads = [&](const Task& tk, TaskLoads& ld) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int row = 32 * wave + 8 * i + (lane >> 3);  // LDS weight row; wavefront row / 32 multiplies it
@@ -218,6 +223,9 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_narrow_kernel(NarrowParams p
       }
       ld.woff[i] = (uint32_t)n * (uint32_t)K + chunk;
     }
+    ld.wbase = p.w + (int64_t)tk.e * p.N * K;
+  };
+  auto setup_token_loads = [&](const TileAux& ax, TaskLoads& ld) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int row = 16 * wave + 8 * i + (lane >> 3);
@@ -226,14 +234,20 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_narrow_kernel(NarrowParams p
       const uint32_t arow = (tok >= 0 && tok < p.P) ? (uint32_t)(tok / p.row_div) : 0u;
       ld.xoff[i] = arow * (uint32_t)K + chunk;
     }
-    ld.wbase = p.w + (int64_t)tk.e * p.N * K;
   };
-  auto issue_stage = [&](const TaskLoads& ld, int stage, int koff) {
+  auto issue_weights = [&](const TaskLoads& ld, int stage, int koff) {
     const uint32_t base = stage0 + stage * kStageBytes;
 #pragma unroll
     for (int i = 0; i < 4; ++i) load_to_lds_16(ld.wbase + koff, ld.woff[i], base + (wave * 4 + i) * 1024);
+  };
+  auto issue_tokens = [&](const TaskLoads& ld, int stage, int koff) {
+    const uint32_t base = stage0 + stage * kStageBytes + kTokOffset;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) load_to_lds_16(p.a_q + koff, ld.xoff[i], base + kTokOffset + (wave * 2 + i) * 1024);
+    for (int i = 0; i < 2; ++i) load_to_lds_16(p.a_q + koff, ld.xoff[i], base + (wave * 2 + i) * 1024);
+  };
+  auto issue_stage = [&](const TaskLoads& ld, int stage, int koff) {
+    issue_weights(ld, stage, koff);
+    issue_tokens(ld, stage, koff);
   };
   // Every wavefront fetches the whole (tiny) set: identical values to identical places, and each
   // wavefront's own wait covers what it reads.
@@ -320,22 +334,27 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_narrow_kernel(NarrowParams p
     }
   };
 
-  // ---- start-up: the first task's inputs, then two steps of loads ----
+  // ---- start-up: the first task's token ids, its weights (which need no ids) behind them, then
+  // what depends on the ids: token rows and scales ----
   int it = blockIdx.x / kXcds;
   Task tk = find_task(it);
   if (tk.e < 0) return;
   int par = 0;
-  issue_ids(tk, aux[0]);
-  wait_vmcnt<0>();
-  __builtin_amdgcn_s_barrier();
   TaskLoads ld;
-  setup_loads(tk, aux[0], ld);
+  issue_ids(tk, aux[0]);
+  setup_weight_loads(tk, ld);
+  issue_weights(ld, 0, 0);
+  issue_weights(ld, 1, kBK);
+  wait_vmcnt<8>();  // the ids are in; every wavefront fetched its own copy, so no barrier is needed
+  setup_token_loads(aux[0], ld);
   issue_scales(tk, aux[0]);
-  issue_stage(ld, 0, 0);
-  issue_stage(ld, 1, kBK);
-  int last_group = kStageLoads;  // size of the most recent group of loads
+  issue_tokens(ld, 0, 0);
+  issue_tokens(ld, 1, kBK);
+  int last_group = kFirstGroup;  // size of the most recent group of loads: the token rows of step 1
   int nit = it + stride;
   Task nx = find_task(nit);
+  int nnit = nit;
+  Task nnx = nx;
   TaskLoads nld = ld;
 
   bool landed = false;  // the loads of the coming step are known to have landed (waited for before the stores)
@@ -362,7 +381,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_narrow_kernel(NarrowParams p
       } else if (s == 2) {
         // they are in (issued two steps ago): the next tile's row addresses and scales
         const Task& t2 = nx.e >= 0 ? nx : tk;
-        setup_loads(t2, aux[par ^ 1], nld);
+        setup_weight_loads(t2, nld);
+        setup_token_loads(aux[par ^ 1], nld);
         issue_scales(t2, aux[par ^ 1]);
         last_group = kStageLoads + aux_loads<MODE>();
       }
@@ -372,6 +392,12 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_narrow_kernel(NarrowParams p
         issue_stage(nld, fill, (s + 2 - nk) * kBK);
       else
         issue_stage(ld, fill, (nk - 1) * kBK);  // nothing left to fetch: keeps the group sizes uniform
+      if (s == 3 && nx.e >= 0) {
+        // The task after the next is looked up here, where the wait for the two scalar loads hides
+        // behind the loads just issued, and not between two tiles.
+        nnit = nit + stride;
+        nnx = find_task(nnit);
+      }
       const char* st = stages + stage * kStageBytes;
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
@@ -393,8 +419,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_narrow_kernel(NarrowParams p
     ld = nld;
     par ^= 1;
     it = nit;
-    nit = it + stride;
-    nx = find_task(nit);
+    nit = nnit;
+    nx = nnx;
   }
   wait_vmcnt<0>();
 }
