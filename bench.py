@@ -30,7 +30,7 @@ if str(ROOT) not in sys.path:
 
 PEAK_INT8_OPS = 5.0e15  # MI355X dense INT8 MFMA, op/s
 PEAK_HBM_BPS = 8.0e12  # MI355X HBM3E, byte/s
-SWEEP_M = (16, 128, 1024, 8192)
+SWEEP_M = (16, 128, 512, 1024, 8192)
 
 
 def _profile_traffic(kernel: str, M: int):
