@@ -62,7 +62,7 @@ struct StreamParams {
   int N;
   int K;
   int B;
-  int pairs_per_wave;  // consecutive tile pairs one wavefront streams back to back
+  int wave_capacity;  // wavefronts of this kernel the device holds at a time
   void* out;
 };
 
@@ -316,24 +316,48 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
   return nvalid;
 }
 
-// grid.x: groups of kWaves wavefronts along the weight rows; grid.y: 64-row (B-row) blocks.
-// NS = sub-tiles per pass.
+// grid.x * grid.y: one workgroup of kWaves wavefronts per kWaves tile pairs and per block of the
+// row list's capacity (grid.z: see below).  NS = sub-tiles per pass.
 template <int MODE, bool kFused, int NS>
 __global__ __launch_bounds__(kThreads, NS == 1 ? 3 : 2) void gemm_stream_kernel(StreamParams p) {
   __shared__ __align__(16) char lds[kWaves * kWaveLds];
   __shared__ __align__(16) char a_lds[kFused ? kSub * (kFusedMaxK + kFusedRowPad) : 16];
   __shared__ float s_lds[kSub];
-  const int blk = blockIdx.y;
   const int npp = *p.npp;
-  if ((int64_t)blk * p.B >= npp) return;
+  const int nblocks = npp / p.B;  // blocks in use: the first ones of the grid's capacity
+  const int total_pairs = MODE == kGateUpSilu ? p.N / 2 / 16 : (p.N / 16 + kTiles - 1) / kTiles;
+  // Consecutive tile pairs a wavefront streams back to back: one (more wavefronts in flight beat
+  // longer streams per wavefront), except where the workgroup quantises the block's rows itself.
+  // Every workgroup of a block repeats that quantisation, so there a wavefront takes 2 or 4 pairs
+  // once the blocks in use need more wavefronts than the device holds at a time anyway.  Known
+  // only here: the number of blocks in use.
+  int ppw = 1;
+  if constexpr (kFused) {
+    const int64_t wanted = (int64_t)nblocks * total_pairs;
+    ppw = wanted > 2 * (int64_t)p.wave_capacity ? 4 : wanted > p.wave_capacity ? 2 : 1;
+  }
+  // With more than one pair per wavefront a block needs fewer workgroups than the grid has for it.
+  // The work is then dealt to the workgroups in the order the device dispatches them (x fastest,
+  // then y), so that the ones with nothing to do are the last ones and the others spread evenly
+  // over the chip's dies and compute units (leaving every block's surplus workgroups idle in place
+  // would starve the dies those land on).
+  int blk = blockIdx.y, group = blockIdx.x;
+  if constexpr (kFused) {
+    const int groups = (total_pairs + kWaves * ppw - 1) / (kWaves * ppw);  // workgroups per block
+    const uint32_t order = blockIdx.x + gridDim.x * blockIdx.y;  // the launcher keeps grid.x * grid.y below 2^31
+    if (order >= (uint32_t)nblocks * (uint32_t)groups) return;
+    blk = (int)(order / (uint32_t)groups);
+    group = (int)(order - (uint32_t)blk * (uint32_t)groups);
+  } else {
+    if (blk >= nblocks) return;
+  }
   const int e = p.expert_ids[blk];
   if (e < 0 || e >= p.E) return;
-  const int total_pairs = MODE == kGateUpSilu ? p.N / 2 / 16 : (p.N / 16 + kTiles - 1) / kTiles;
-  const int first_pair = (blockIdx.x * kWaves + threadIdx.x / kWave) * p.pairs_per_wave;
+  const int first_pair = (group * kWaves + threadIdx.x / kWave) * ppw;
   // a wavefront past the last weight rows leaves, unless the workgroup needs it for the quantisation
   if (!kFused && first_pair >= total_pairs) return;
   const int left = total_pairs - first_pair;
-  const int npairs = left < 0 ? 0 : left < p.pairs_per_wave ? left : p.pairs_per_wave;
+  const int npairs = left < 0 ? 0 : left < ppw ? left : ppw;
 
   char* wave_lds = lds + (threadIdx.x / kWave) * kWaveLds;
   if (gridDim.z > 1) {
@@ -353,6 +377,16 @@ __global__ __launch_bounds__(kThreads, NS == 1 ? 3 : 2) void gemm_stream_kernel(
   const int nsub = (nvalid + kSub - 1) / kSub;
   for (int sub0 = NS; sub0 < nsub; sub0 += NS)
     stream_pass<MODE, NS, kFused>(p, blk, e, sub0, first_pair, npairs, wave_lds, false, a_lds, s_lds);
+}
+
+int device_cu_count() {
+  static const int count = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) return 256;
+    return n;
+  }();
+  return count;
 }
 
 template <int MODE, bool kFused = false>
@@ -375,14 +409,10 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   p.B = a.block_size;
   p.out = a.out;
   const int total_pairs = MODE == kGateUpSilu ? a.n / 2 / 16 : (a.n / 16 + kTiles - 1) / kTiles;
-  // One tile pair per wavefront measured best in the decode regime (more wavefronts in flight beat
-  // longer streams per wavefront); the kernel itself handles any number of consecutive pairs.
-  const int ppw = 1;
-  p.pairs_per_wave = ppw;
-  const int waves = (total_pairs + ppw - 1) / ppw;
+  const int waves = total_pairs;  // the kernel groups pairs per wavefront once it knows the blocks in use
   const int64_t blocks = (a.sorted_cap + a.block_size - 1) / a.block_size;
   if (blocks == 0 || waves == 0) return hipSuccess;
-  if (blocks > 65535) return hipErrorInvalidValue;
+  if (blocks > 65535 || blocks * ((waves + kWaves - 1) / kWaves) >= (1ll << 31)) return hipErrorInvalidValue;
   const bool two = !kFused && a.num_pairs > (int64_t)kPairRowsPerExpert * a.num_experts;
   // Passes per block that can be needed: no expert holds more rows than there are tokens (or pairs,
   // when the caller did not say).  One workgroup per pass once there can be more than one.
@@ -392,6 +422,7 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   const int64_t rows = most_rows < a.block_size ? most_rows : a.block_size;
   const int passes = kFused ? 1 : (int)((rows + kSub * ns - 1) / (kSub * ns));
   const dim3 grid((unsigned)((waves + kWaves - 1) / kWaves), (unsigned)blocks, (unsigned)(passes > 1 ? passes : 1));
+  p.wave_capacity = device_cu_count() * kWaves * (two ? 2 : 3);
   if (two)
     hipLaunchKernelGGL((gemm_stream_kernel<MODE, kFused, kFused ? 1 : 2>), grid, dim3(kThreads), 0, stream, p);
   else
