@@ -49,7 +49,7 @@ int check_gemm_common(const void* a_q, const void* w, const int32_t* sorted, con
   return MOE_I8_OK;
 }
 
-constexpr int kStreamRowsPerExpert = 12;
+constexpr int kStreamRowsPerExpert = 8;
 constexpr int kNarrowRowsPerExpert = 56;
 
 // Which family a launch goes to (one of the MOE_I8_GEMM_* constants, never AUTO); -1 with the error
@@ -66,9 +66,13 @@ int picks_family(const moe_i8::GemmArgs& g, int variant) {
     return MOE_I8_GEMM_NARROW;
   }
   if (variant == MOE_I8_GEMM_STREAM) return MOE_I8_GEMM_STREAM;
-  // Measured crossovers on the Qwen3-30B-A3B shape, in routed rows per expert: the streaming family
-  // wins while a block mostly holds one 16-row sub-tile (up to about 12), the narrow tiles while
-  // most experts hold a single 64-row block (up to about 56), the wide LDS tiles beyond.
+  // Measured crossovers on the Qwen3-30B-A3B shape, in routed rows per expert: with evenly spread
+  // routing the streaming family wins while a block mostly holds one 16-row sub-tile (up to about
+  // 12), the narrow tiles while most experts hold a single 64-row block (up to about 56), the wide
+  // LDS tiles beyond.  The streaming family reads an expert's weights once per 16 (or 32) of its
+  // rows, so skewed routing costs it far more than the tiled families (a few experts with a
+  // hundred rows double its time); the first crossover is therefore set lower, at 8, where the
+  // narrow tiles lose 2 % or less on even routing.
   const int64_t rows_x_experts = g.num_pairs;
   if (rows_x_experts <= (int64_t)kStreamRowsPerExpert * g.num_experts) return MOE_I8_GEMM_STREAM;
   if (rows_x_experts <= (int64_t)kNarrowRowsPerExpert * g.num_experts && moe_i8::gemm_narrow_supports(g))
