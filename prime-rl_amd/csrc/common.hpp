@@ -14,6 +14,17 @@ constexpr int kMaxExperts = 1024;  // == MOE_I8_MAX_EXPERTS
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 
+// Compute units of the current device (asked once per process; 256 if the runtime will not say).
+inline int device_cu_count() {
+  static const int count = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8) return 256;
+    return n;
+  }();
+  return count;
+}
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 
 // fp32 -> bf16 bits, round to nearest even; NaN stays a quiet NaN.

@@ -425,16 +425,6 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_narrow_kernel(NarrowParams p
   wait_vmcnt<0>();
 }
 
-int device_cu_count() {
-  static const int count = [] {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 256;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < kXcds) return 256;
-    return n;
-  }();
-  return count;
-}
-
 template <int MODE>
 hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   NarrowParams p;

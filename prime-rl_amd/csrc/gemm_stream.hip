@@ -379,16 +379,6 @@ __global__ __launch_bounds__(kThreads, NS == 1 ? 3 : 2) void gemm_stream_kernel(
     stream_pass<MODE, NS, kFused>(p, blk, e, sub0, first_pair, npairs, wave_lds, false, a_lds, s_lds);
 }
 
-int device_cu_count() {
-  static const int count = [] {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 256;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) return 256;
-    return n;
-  }();
-  return count;
-}
-
 template <int MODE, bool kFused = false>
 hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   StreamParams p;
