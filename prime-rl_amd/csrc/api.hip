@@ -295,12 +295,13 @@ int moe_i8_quant_weights(const void* w, int dtype, int64_t rows, int64_t cols, i
   return check_launch(moe_i8::launch_quant_weights(a, static_cast<hipStream_t>(stream)), "quant_weights");
 }
 
-int moe_i8_gemm_gate_up_silu(const int8_t* x_q, const float* a_scale, const int8_t* w1,
-                             const float* w1_scale, const int32_t* sorted_token_ids,
-                             const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
-                             int64_t num_pairs, int top_k, int num_experts, int hidden, int inter,
-                             int block_size, int64_t sorted_cap, void* act_out, int variant,
-                             void* stream) {
+// The gate_up GEMM behind the entry point; `from_align`: the routing arrays are moe_align's own
+// output (the caller of the entry point may pass anything).
+static int gemm_gate_up_impl(const int8_t* x_q, const float* a_scale, const int8_t* w1, const float* w1_scale,
+                             const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                             const int32_t* num_tokens_post_padded, int64_t num_pairs, int top_k, int num_experts,
+                             int hidden, int inter, int block_size, int64_t sorted_cap, void* act_out, int variant,
+                             bool from_align, void* stream) {
   if (num_pairs == 0) return MOE_I8_OK;
   if (inter < 16 || inter % 16 || inter > (1 << 29)) return fail(MOE_I8_EINVAL, "inter (%d) must be a positive multiple of 16", inter);
   if (int rc = check_gemm_common(x_q, w1, sorted_token_ids, expert_ids, num_tokens_post_padded,
@@ -329,15 +330,27 @@ int moe_i8_gemm_gate_up_silu(const int8_t* x_q, const float* a_scale, const int8
   g.sorted_cap = sorted_cap;
   g.out = act_out;
   g.max_rows_per_expert = (num_pairs + top_k - 1) / top_k;  // an expert sees a token at most once
+  g.expert_ids_ascend = from_align;
   return run_gemm(g, variant, static_cast<hipStream_t>(stream));
 }
 
-// The down GEMM behind the entry point; `max_rows` bounds the rows any one expert can hold (0: unknown).
+int moe_i8_gemm_gate_up_silu(const int8_t* x_q, const float* a_scale, const int8_t* w1,
+                             const float* w1_scale, const int32_t* sorted_token_ids,
+                             const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
+                             int64_t num_pairs, int top_k, int num_experts, int hidden, int inter,
+                             int block_size, int64_t sorted_cap, void* act_out, int variant,
+                             void* stream) {
+  return gemm_gate_up_impl(x_q, a_scale, w1, w1_scale, sorted_token_ids, expert_ids, num_tokens_post_padded, num_pairs,
+                           top_k, num_experts, hidden, inter, block_size, sorted_cap, act_out, variant, false, stream);
+}
+
+// The down GEMM behind the entry point; `max_rows` bounds the rows any one expert can hold (0: unknown),
+// `from_align` as above.
 static int gemm_down_impl(const int8_t* h_q, const float* a_scale, const int8_t* w2, const float* w2_scale,
                           const float* topk_weights, const int32_t* sorted_token_ids, const int32_t* expert_ids,
                           const int32_t* num_tokens_post_padded, int64_t num_pairs, int num_experts, int hidden,
                           int inter, int block_size, int64_t sorted_cap, void* out, int variant, int64_t max_rows,
-                          void* stream) {
+                          bool from_align, void* stream) {
   if (num_pairs == 0) return MOE_I8_OK;
   if (int rc = check_gemm_common(h_q, w2, sorted_token_ids, expert_ids, num_tokens_post_padded, out,
                                  num_pairs, num_experts, hidden, inter, block_size, sorted_cap,
@@ -349,6 +362,7 @@ static int gemm_down_impl(const int8_t* h_q, const float* a_scale, const int8_t*
                                  num_tokens_post_padded, num_pairs, num_experts, hidden, inter, block_size,
                                  sorted_cap, out);
   g.max_rows_per_expert = max_rows;
+  g.expert_ids_ascend = from_align;
   return run_gemm(g, variant, static_cast<hipStream_t>(stream));
 }
 
@@ -360,7 +374,7 @@ int moe_i8_gemm_down(const int8_t* h_q, const float* a_scale, const int8_t* w2,
                      int variant, void* stream) {
   return gemm_down_impl(h_q, a_scale, w2, w2_scale, topk_weights, sorted_token_ids, expert_ids,
                         num_tokens_post_padded, num_pairs, num_experts, hidden, inter, block_size, sorted_cap, out,
-                        variant, 0, stream);
+                        variant, 0, false, stream);
 }
 
 int moe_i8_gemm_down_bf16(const void* act, const int8_t* w2, const float* w2_scale, const float* topk_weights,
@@ -529,14 +543,15 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
                                          npp, ws + c.align_ws, c.align_bytes, stream))
       return rc;
   }
-  if (int rc = moe_i8_gemm_gate_up_silu(x_q, a1, w1, w1_scale, sorted, eids, npp, p, top_k, num_experts,
-                                        hidden_size, inter, block_size, c.cap, act, variant, stream))
+  if (int rc = gemm_gate_up_impl(x_q, a1, w1, w1_scale, sorted, eids, npp, p, top_k, num_experts, hidden_size, inter,
+                                 block_size, c.cap, act, variant, true, stream))
     return rc;
   // Very few rows per expert (decode): the streaming down GEMM quantises its activations itself, one
   // launch less.  Every workgroup of a block repeats that quantisation, so from about four rows
   // per expert on (measured) the separate launch is the cheaper one again.
-  const moe_i8::GemmArgs dg = down_args(act_q, a2, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
-                                        hidden_size, inter, block_size, c.cap, down);
+  moe_i8::GemmArgs dg = down_args(act_q, a2, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
+                                  hidden_size, inter, block_size, c.cap, down);
+  dg.expert_ids_ascend = true;
   const int down_family = picks_family(dg, variant);
   if (down_family < 0) return MOE_I8_EUNSUPPORTED;
   if (down_family == MOE_I8_GEMM_STREAM && moe_i8::gemm_stream_fuses_quant(inter) && p <= (int64_t)3 * num_experts) {
@@ -547,7 +562,7 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
     if (int rc = moe_i8_quant_rows(act, MOE_I8_DTYPE_BF16, p, inter, inter, nullptr, 1, p, act_q, a2, stream))
       return rc;
     if (int rc = gemm_down_impl(act_q, a2, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
-                                hidden_size, inter, block_size, c.cap, down, variant, m, stream))
+                                hidden_size, inter, block_size, c.cap, down, variant, m, true, stream))
       return rc;
   }
   return moe_i8_sum(down, out, m, top_k, hidden_size, stream);

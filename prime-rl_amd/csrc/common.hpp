@@ -199,6 +199,7 @@ struct GemmArgs {
   int64_t sorted_cap;
   void* out;  // bf16 [P, I] | bf16 [P, H] | int32 [P, N]
   int64_t max_rows_per_expert = 0;  // upper bound if the caller knows one (the token count), else 0
+  bool expert_ids_ascend = false;   // expert_ids is known to come from moe_align (non-decreasing over the used blocks)
 };
 hipError_t launch_gemm_stream(const GemmArgs& a, hipStream_t stream);
 // register-only int8 MFMA loop (measurement aid): sink holds mfma_probe_sink_bytes(workgroups)

@@ -539,9 +539,16 @@ bool gemm_tile_supports(const GemmArgs& a) {
   // per-lane source offsets are 32-bit: one expert's weights and the activation matrix must each
   // span less than 4 GiB
   const int64_t act_rows = (a.num_pairs + a.row_div - 1) / a.row_div;
-  return (a.block_size == 64 || a.block_size == 128) && a.k % kBK == 0 && a.k >= 2 * kBK && a.n % 16 == 0 &&
-         (a.sorted_cap + a.block_size - 1) / a.block_size <= kMaxTiles && (int64_t)a.n * a.k < (1ll << 32) &&
-         act_rows * a.k < (1ll << 32);
+  if (!((a.block_size == 64 || a.block_size == 128) && a.k % kBK == 0 && a.k >= 2 * kBK && a.n % 16 == 0 &&
+        (int64_t)a.n * a.k < (1ll << 32) && act_rows * a.k < (1ll << 32)))
+    return false;
+  // The tile list lives in LDS.  A run of equal expert ids of L blocks makes ceil(L / blocks per
+  // tile) tiles; moe_align's ids ascend, so there is one run per expert.  Ids of unknown order could
+  // make every block a tile of its own.  While the list is built the block ids sit in the stages.
+  const int64_t blocks = (a.sorted_cap + a.block_size - 1) / a.block_size;
+  const int per_tile = kTileTok / a.block_size;
+  const int64_t tiles = a.expert_ids_ascend ? (blocks + per_tile - 1) / per_tile + a.num_experts : blocks;
+  return tiles <= kMaxTiles && blocks <= (int64_t)(2 * kStageBytes / sizeof(int)) && blocks <= 65535;
 }
 
 hipError_t launch_gemm_tile(const GemmArgs& a, hipStream_t stream) {

@@ -44,7 +44,7 @@ def test_fused_experts_matches_oracle(pra, oracle, shape_name, M, variant):
 
 
 @pytest.mark.parametrize("shape_name,M,weights_on_device", [
-    ("qwen3-30b-a3b", 8192, False), ("glm-4.5-air", 512, False), ("glm-4.5-air", 4096, False),
+    ("qwen3-30b-a3b", 8192, False), ("qwen3-30b-a3b", 65536, True), ("glm-4.5-air", 512, False), ("glm-4.5-air", 4096, False),
     ("deepseek-v3", 8, True), ("deepseek-v3", 64, True), ("deepseek-v3", 2048, True), ("deepseek-v3", 16384, True),
 ])
 def test_fused_experts_full_size_sampled_tokens(pra, oracle, shape_name, M, weights_on_device):
