@@ -401,26 +401,6 @@ hipError_t launch_align_quant(const AlignArgs& a, const QuantArgs& q, hipStream_
   return hipGetLastError();
 }
 
-// Routing of a dense layer seen as one expert that every row visits: rows in order, padded to a
-// whole block with the sentinel, every used block owned by expert 0, the rest of both arrays
-// (capacities as moe_align would leave them) marked unused.
-__global__ void identity_routing_kernel(int rows, int block_size, int64_t sorted_cap, int32_t* __restrict__ sorted,
-                                        int32_t* __restrict__ expert_ids, int32_t* __restrict__ npp_out) {
-  const int padded = (rows + block_size - 1) / block_size * block_size;
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < sorted_cap) sorted[i] = i < rows ? (int32_t)i : rows;
-  if (i < (sorted_cap + block_size - 1) / block_size) expert_ids[i] = i < padded / block_size ? 0 : -1;
-  if (i == 0) *npp_out = padded;
-}
-
-hipError_t launch_identity_routing(int rows, int block_size, int64_t sorted_cap, int32_t* sorted,
-                                   int32_t* expert_ids, int32_t* npp, hipStream_t stream) {
-  const int threads = 256;
-  hipLaunchKernelGGL(identity_routing_kernel, dim3((unsigned)(sorted_cap > 0 ? (sorted_cap + threads - 1) / threads : 1)),
-                     dim3(threads), 0, stream, rows, block_size, sorted_cap, sorted, expert_ids, npp);
-  return hipGetLastError();
-}
-
 hipError_t launch_align(const AlignArgs& a, hipStream_t stream) {
   const int E = a.num_experts;
   const int nbits = bits_for(E);

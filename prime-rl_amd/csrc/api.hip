@@ -573,6 +573,7 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
 //   (mlp only) act bf16[M*I] | act_q i8[M*I] | a2 f32[M]
 namespace {
 constexpr int kDenseBlock = 64;
+constexpr int kDenseSelfQuantRows = 16;  // up to this many rows the down GEMM of the MLP quantises its own input
 struct DenseCarve {
   int64_t x_q, a1, sorted, eids, npp, act, act_q, a2, total, cap;
 };
@@ -606,14 +607,26 @@ int dense_prologue(const void* x, int64_t m, int k, void* workspace, int64_t wor
   if (workspace_bytes < c.total)
     return fail(MOE_I8_EWORKSPACE, "workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)c.total);
   char* ws = static_cast<char*>(workspace);
-  if (int rc = moe_i8_scaled_int8_quant(x, MOE_I8_DTYPE_BF16, m, k, k, reinterpret_cast<int8_t*>(ws + c.x_q),
-                                        reinterpret_cast<float*>(ws + c.a1), stream))
-    return rc;
-  return check_launch(
-      moe_i8::launch_identity_routing((int)m, kDenseBlock, c.cap, reinterpret_cast<int32_t*>(ws + c.sorted),
-                                      reinterpret_cast<int32_t*>(ws + c.eids),
-                                      reinterpret_cast<int32_t*>(ws + c.npp), static_cast<hipStream_t>(stream)),
-      "identity_routing");
+  // one launch: the ties-to-even row quantiser, whose threads also write the identity routing
+  if (k < 8 || k % 8) return fail(MOE_I8_EINVAL, "k (%d) must be a positive multiple of 8", k);
+  if (!aligned16(x)) return fail(MOE_I8_EINVAL, "x must be 16-byte aligned");
+  moe_i8::QuantArgs a;
+  a.x = static_cast<const uint16_t*>(x);
+  a.src_rows = m;
+  a.cols = k;
+  a.row_stride = k;
+  a.gather = nullptr;
+  a.gather_div = 1;
+  a.rows = m;
+  a.q = reinterpret_cast<int8_t*>(ws + c.x_q);
+  a.scale = reinterpret_cast<float*>(ws + c.a1);
+  a.round_even = 1;
+  a.route_sorted = reinterpret_cast<int32_t*>(ws + c.sorted);
+  a.route_expert_ids = reinterpret_cast<int32_t*>(ws + c.eids);
+  a.route_npp = reinterpret_cast<int32_t*>(ws + c.npp);
+  a.route_block = kDenseBlock;
+  a.route_cap = c.cap;
+  return check_launch(moe_i8::launch_quant_rows(a, static_cast<hipStream_t>(stream)), "quant_rows");
 }
 }  // namespace
 
@@ -656,6 +669,24 @@ int moe_i8_w8a8_mlp(const void* x, const int8_t* w13, const float* w13_scale, co
   if (int rc = moe_i8_gemm_gate_up_silu(x_q, a1, w13, w13_scale, sorted, eids, npp, m, 1, 1, hidden, inter,
                                         kDenseBlock, c.cap, ws + c.act, variant, stream))
     return rc;
+  // A few rows (decode): the streaming down GEMM quantises them itself (ties to even here), one
+  // launch less.
+  moe_i8::GemmArgs dg = down_args(act_q, a2, w2, w2_scale, nullptr, sorted, eids, npp, m, 1, hidden, inter,
+                                  kDenseBlock, c.cap, out);
+  dg.expert_ids_ascend = true;
+  const int family = picks_family(dg, variant);
+  if (family < 0) return MOE_I8_EUNSUPPORTED;
+  if (family == MOE_I8_GEMM_STREAM && m <= kDenseSelfQuantRows && moe_i8::gemm_stream_fuses_quant(inter)) {
+    if (int rc = check_gemm_common(ws + c.act, w2, sorted, eids, npp, out, m, 1, hidden, inter, kDenseBlock, c.cap,
+                                   MOE_I8_GEMM_STREAM))
+      return rc;
+    if (!aligned16(w2_scale)) return fail(MOE_I8_EINVAL, "w2_scale must be 16-byte aligned");
+    dg.a_q = nullptr;
+    dg.a_scale = nullptr;
+    dg.a_bf16 = reinterpret_cast<const uint16_t*>(ws + c.act);
+    dg.a_round_even = true;
+    return check_launch(moe_i8::launch_gemm_stream(dg, static_cast<hipStream_t>(stream)), "gemm_stream");
+  }
   if (int rc = moe_i8_scaled_int8_quant(ws + c.act, MOE_I8_DTYPE_BF16, m, inter, inter, act_q, a2, stream)) return rc;
   return moe_i8_gemm_down(act_q, a2, w2, w2_scale, nullptr, sorted, eids, npp, m, 1, hidden, inter, kDenseBlock,
                           c.cap, out, variant, stream);

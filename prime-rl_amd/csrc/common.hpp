@@ -143,6 +143,14 @@ struct QuantArgs {
   int64_t out_rows_per_group = 0;
   int64_t out_row_offset = 0;
   int round_even = 0;  // activations: ties to even instead of away from zero
+  // Row quantiser only: also write the routing of a dense layer seen as one expert that every row
+  // visits (rows in order, padded to whole blocks with the sentinel, used blocks owned by expert
+  // 0, the rest of both arrays marked unused) — one launch less in front of a dense GEMM.
+  int32_t* route_sorted = nullptr;  // null: no routing
+  int32_t* route_expert_ids = nullptr;
+  int32_t* route_npp = nullptr;
+  int route_block = 0;
+  int64_t route_cap = 0;
 };
 hipError_t launch_quant_rows(const QuantArgs& a, hipStream_t stream);
 // Router: scores -> (grouped) top-k -> weights, one wavefront per token.
@@ -172,8 +180,6 @@ hipError_t launch_route_topk(const RouteArgs& a, hipStream_t stream);
 // Per-output-channel weight quantisation (round to nearest even of w / scale, scale = absmax / 127).
 hipError_t launch_quant_weights(const QuantArgs& a, hipStream_t stream);
 // moe_align and the quantisation of `q` in one launch; only when align_quant_fusable() says so.
-hipError_t launch_identity_routing(int rows, int block_size, int64_t sorted_cap, int32_t* sorted,
-                                   int32_t* expert_ids, int32_t* npp, hipStream_t stream);
 bool align_quant_fusable(const AlignArgs& a, const QuantArgs& q);
 hipError_t launch_align_quant(const AlignArgs& a, const QuantArgs& q, hipStream_t stream);
 
@@ -182,6 +188,7 @@ enum GemmMode { kGateUpSilu = 0, kDown = 1, kAccI32 = 2 };
 struct GemmArgs {
   int mode;
   const uint16_t* a_bf16 = nullptr;  // down, streaming family only: bf16 activations [P, K] quantised in the kernel
+  bool a_round_even = false;         // ... rounding ties to even (dense path) instead of away from zero (MoE path)
   const int8_t* a_q;      // [*, K] activations (int8)
   const float* a_scale;   // per activation row
   const int8_t* w;        // [E, N, K]

@@ -63,6 +63,7 @@ struct StreamParams {
   int K;
   int B;
   int wave_capacity;  // wavefronts of this kernel the device holds at a time
+  int round_even;     // in-kernel quantisation: ties to even instead of away from zero
   void* out;
 };
 
@@ -181,7 +182,9 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
 #pragma unroll
       for (int c = 0; c < kFusedMaxK / kQuantVec / kWave; ++c) {
         const int idx = lane + c * kWave;
-        if (idx < nvec) *reinterpret_cast<uint2*>(a_lds + r * row_bytes + idx * 8) = quant8(v[c], inv);
+        if (idx < nvec)
+          *reinterpret_cast<uint2*>(a_lds + r * row_bytes + idx * 8) =
+              p.round_even ? quant8<true>(v[c], inv) : quant8<false>(v[c], inv);
       }
     }
     __syncthreads();
@@ -413,6 +416,7 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   const int passes = kFused ? 1 : (int)((rows + kSub * ns - 1) / (kSub * ns));
   const dim3 grid((unsigned)((waves + kWaves - 1) / kWaves), (unsigned)blocks, (unsigned)(passes > 1 ? passes : 1));
   p.wave_capacity = device_cu_count() * kWaves * (two ? 2 : 3);
+  p.round_even = a.a_round_even ? 1 : 0;
   if (two)
     hipLaunchKernelGGL((gemm_stream_kernel<MODE, kFused, kFused ? 1 : 2>), grid, dim3(kThreads), 0, stream, p);
   else

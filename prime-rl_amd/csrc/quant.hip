@@ -22,6 +22,18 @@ template <int VPL, int kMode>
 __global__ __launch_bounds__(kThreads) void quant_rows_kernel(QuantArgs a) {
   const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
   if (row < a.rows) quant_one_row<VPL, kMode>(a, row);
+  if (a.route_sorted != nullptr) {
+    // identity routing of a.rows rows, written by all threads of the launch in strides
+    const int rows = (int)a.rows;
+    const int padded = (rows + a.route_block - 1) / a.route_block * a.route_block;
+    const int64_t blocks_cap = (a.route_cap + a.route_block - 1) / a.route_block;
+    const int64_t step = (int64_t)gridDim.x * kThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < a.route_cap; i += step) {
+      a.route_sorted[i] = i < rows ? (int32_t)i : rows;
+      if (i < blocks_cap) a.route_expert_ids[i] = i < padded / a.route_block ? 0 : -1;
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) *a.route_npp = padded;
+  }
 }
 
 template <int kMode>

@@ -83,3 +83,19 @@ def test_gated_mlp(pra, oracle, variant, M, H, I):
                             per_channel_quant=True, w1_scale=s13.to(DEV)[None], w2_scale=s2.to(DEV)[None],
                             gemm_variant=variant)
     assert rel_err(out.cpu(), moe.cpu()) < 5e-3
+
+
+@pytest.mark.parametrize("m", [1, 7, 16])
+@pytest.mark.parametrize("H,I", [(2048, 768), (256, 128), (4096, 1024)])
+def test_gated_mlp_of_a_few_rows_equals_the_rows_of_a_larger_call(pra, H, I, m):
+    """Up to 16 rows the MLP runs as three launches (the down GEMM quantises its own input, ties to
+    even); rows are independent, so the result must be, bit for bit, what the same rows give inside a
+    larger call that takes the five-launch path."""
+    g = torch.Generator().manual_seed(m + I)
+    x = torch.randn(96, H, generator=g).to(torch.bfloat16).to(DEV)
+    w13, s13 = _weights(2 * I, H, g)
+    w2, s2 = _weights(H, I, g)
+    args = (w13.to(DEV), (s13 * 0.3).to(DEV), w2.to(DEV), (s2 * 0.3).to(DEV))
+    big = pra.w8a8_mlp(x, *args)
+    small = pra.w8a8_mlp(x[:m].contiguous(), *args)
+    assert torch.equal(small, big[:m]), int((small != big[:m]).sum())
