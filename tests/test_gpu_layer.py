@@ -115,12 +115,13 @@ def test_block_size_does_not_change_the_result(pra):
         assert torch.equal(ref, _run(pra, inp, block_size_m=B))
 
 
-def test_hip_graph_replay(pra):
+@pytest.mark.parametrize("M", [16, 512, 2048])  # streaming, narrow-tile and wide-tile GEMM families
+def test_hip_graph_replay(pra, M):
     """The call records no allocation, memset or synchronisation, so it can be captured and replayed."""
     im = inputs_mod()
-    inp = im.make_inputs("qwen3-30b-a3b", 16, seed=4).to(DEV)
+    inp = im.make_inputs("qwen3-30b-a3b", M, seed=4).to(DEV)
     eager = _run(pra, inp)
-    ws = torch.empty((pra.workspace_bytes(16, 8, 128, 2048, 768, 64),), dtype=torch.uint8, device=DEV)
+    ws = torch.empty((pra.workspace_bytes(M, 8, 128, 2048, 768, 64),), dtype=torch.uint8, device=DEV)
     static_x = inp.hidden_states.clone()
     out = torch.empty_like(static_x)
     kw = dict(workspace=ws, **inp.fused_experts_kwargs())
