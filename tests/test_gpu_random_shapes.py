@@ -30,6 +30,20 @@ def _cases():
             M = max(1, int(1.5e10 / (k * I * H)))
         routing = rng.choice(["softmax", "softmax", "zipf"])
         cases.append((i, E, k, H, I, M, B, routing))
+    # shapes every GEMM family supports (reduction lengths that are multiples of 128 and at least 512,
+    # blocks of 64 or 128 rows), around the rows-per-expert counts where the families hand over
+    for i in range(120, 170):
+        E = rng.choice([3, 8, 16, 40])
+        k = min(rng.choice([1, 2, 4, 8]), E)
+        H = rng.choice([512, 640, 1024, 1408, 2048])
+        I = rng.choice([512, 640, 768, 1024, 1408])
+        B = rng.choice([64, 64, 128])
+        rows_per_expert = rng.choice([5, 9, 20, 40, 57, 64, 70, 130, 200])
+        M = max(1, int(rows_per_expert * E / k))
+        if M * k * I * H > 1.5e10:
+            M = max(1, int(1.5e10 / (k * I * H)))
+        routing = rng.choice(["softmax", "zipf"])
+        cases.append((i, E, k, H, I, M, B, routing))
     return cases
 
 
