@@ -76,6 +76,23 @@ def time_layer(pkg, torch, dev, weights, steps: int, warmup: int, variant: str) 
     return (time.perf_counter() - t0) / steps
 
 
+def layer_percentiles(pkg, torch, dev, weights, steps: int, variant: str) -> dict:
+    """Spread of the single-call duration: an event pair around every call (the mean of these reads a
+    little above the back-to-back figure, which overlaps host work with the device)."""
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    torch.cuda.synchronize()
+    for i, (a, b) in enumerate(pairs):
+        w1, w2, s1, s2 = weights[i % len(weights)]
+        a.record()
+        pkg.fused_experts(dev.hidden_states, w1, w2, dev.topk_weights, dev.topk_ids, use_int8_w8a8=True,
+                          per_channel_quant=True, w1_scale=s1, w2_scale=s2, gemm_variant=variant)
+        b.record()
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) * 1e3 for a, b in pairs)
+    pick = lambda q: ts[min(len(ts) - 1, int(q * len(ts)))]
+    return {"p10": pick(0.10), "p50": pick(0.50), "p90": pick(0.90)}
+
+
 def time_gate_up_kernel(pkg, torch, shape, dev, weights, steps: int, warmup: int, variant: str) -> float:
     """Average duration (s) of the gate_up GEMM launch, from event pairs on the launch stream."""
     M, k = dev.topk_ids.shape
@@ -230,6 +247,105 @@ def time_router(pkg, torch, shape, M: int, steps: int, warmup: int) -> dict:
     return {"M": M, "us": t * 1e6, "bytes": nbytes, "hbm_gbps": nbytes / t / 1e9}
 
 
+DECODE_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 160, 192, 224, 256)
+
+
+def time_decode_mix(pkg, torch, shape_name: str, layers: int, steps: int) -> dict:
+    """Continuous-batching decode: `layers` independently seeded layers of the shape called back to back,
+    `steps` steps whose batch size is drawn uniformly from 1..256, routing re-drawn for every step and
+    layer, every layer fed a fresh N(0,1) input (chaining random layers would overflow bf16 within a few
+    layers).  Two ways: eager calls with the true batch size, and HIP-graph replays of the whole stack
+    captured once per batch-size bucket with the batch padded up to the bucket (padding rows are routed
+    like row 0 and thrown away) — the way a serving engine replays captured graphs.  Tokens per second
+    count real tokens only."""
+    shape = pkg.inputs.SHAPES[shape_name]
+    E, k, H, I = shape.E_total, shape.k + (1 if shape.shared_expert else 0), shape.H, shape.I
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(5)
+    stack = []
+    for _ in range(layers):
+        stack.append((torch.randint(-127, 128, (E, 2 * I, H), generator=g, dtype=torch.int8, device=dev),
+                      torch.randint(-127, 128, (E, H, I), generator=g, dtype=torch.int8, device=dev),
+                      torch.empty(E, 2 * I, device=dev).uniform_(0.002, 0.01, generator=g),
+                      torch.empty(E, H, device=dev).uniform_(0.002, 0.01, generator=g)))
+    cpu = torch.Generator().manual_seed(6)
+    max_m = DECODE_BUCKETS[-1]
+    sizes = torch.randint(1, max_m + 1, (steps,), generator=cpu).tolist()
+    n_tables = 64  # routing tables and inputs drawn beforehand, walked cyclically by (step, layer)
+    tables = [tuple(t.to(dev) for t in pkg.inputs.route(shape, max_m, cpu)) for _ in range(n_tables)]
+    xs = [torch.randn(max_m, H, generator=cpu).to(torch.bfloat16).to(dev) for _ in range(8)]
+    ws = torch.empty(pkg.workspace_bytes(max_m, k, E, H, I, 64), dtype=torch.uint8, device=dev)
+    kw = dict(use_int8_w8a8=True, per_channel_quant=True, workspace=ws)
+
+    def eager_step(t, M):
+        for l, (w1, w2, s1, s2) in enumerate(stack):
+            tw, ids = tables[(t * layers + l) % n_tables]
+            pkg.fused_experts(xs[(t + l) % len(xs)][:M], w1, w2, tw[:M], ids[:M], w1_scale=s1, w2_scale=s2, **kw)
+
+    for t in range(3):
+        eager_step(t, sizes[t])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t, M in enumerate(sizes):
+        eager_step(t, M)
+    torch.cuda.synchronize()
+    eager = time.perf_counter() - t0
+
+    # graphs: static inputs per bucket; the routing of every layer is refreshed by device copies before a replay
+    static_x = torch.zeros(max_m, H, dtype=torch.bfloat16, device=dev)
+    static_tw = torch.zeros(layers, max_m, k, dtype=torch.float32, device=dev)
+    static_ids = torch.zeros(layers, max_m, k, dtype=torch.int32, device=dev)
+    all_tw = torch.stack([t[0] for t in tables])   # [n_tables, max_m, k]
+    all_ids = torch.stack([t[1] for t in tables])
+    graphs = {}
+    side = torch.cuda.Stream()
+    for b in DECODE_BUCKETS:
+        def run_stack():
+            for l, (w1, w2, s1, s2) in enumerate(stack):
+                pkg.fused_experts(static_x[:b], w1, w2, static_tw[l, :b], static_ids[l, :b], w1_scale=s1, w2_scale=s2, **kw)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            run_stack()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run_stack()
+        graphs[b] = graph
+    order = torch.arange(layers, device=dev)
+
+    def graph_step(t, M):
+        b = next(x for x in DECODE_BUCKETS if x >= M)
+        idx = (t * layers + order) % n_tables
+        static_tw.copy_(all_tw[idx])
+        static_ids.copy_(all_ids[idx])
+        if M < b:  # padding rows follow row 0's routing
+            static_tw[:, M:b] = static_tw[:, :1]
+            static_ids[:, M:b] = static_ids[:, :1]
+        static_x[:M].copy_(xs[t % len(xs)][:M])
+        graphs[b].replay()
+
+    for t in range(3):
+        graph_step(t, sizes[t])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t, M in enumerate(sizes):
+        graph_step(t, M)
+    torch.cuda.synchronize()
+    replay = time.perf_counter() - t0
+    tokens = sum(sizes)
+    small = sum(1 for M in sizes if M * k <= 3 * E)
+    del stack, graphs
+    torch.cuda.empty_cache()
+    return {"shape": shape_name, "layers": layers, "steps": steps, "tokens": tokens,
+            "batch_sizes": f"uniform 1..{max_m}, mean {tokens / steps:.1f}",
+            "eager": {"wall_s": eager, "tokens_per_s": tokens / eager, "us_per_layer_call": eager / (steps * layers) * 1e6},
+            "hip_graph": {"wall_s": replay, "tokens_per_s": tokens / replay,
+                          "us_per_layer_call": replay / (steps * layers) * 1e6, "buckets": list(DECODE_BUCKETS),
+                          "note": "one captured graph of the whole stack per bucket; batch padded up to the bucket; "
+                                  "includes the device copies that refresh inputs and routing"},
+            "launches_per_layer": {"4 (down GEMM quantises its own input)": small, "5": steps - small}}
+
+
 def time_mfma_ceiling(pkg, torch) -> dict:
     """What the device sustains on a register-only int8 MFMA loop (no memory traffic at all) with constant
     and with pseudo-random operand bits: the board's power limit lowers the clock as the operand bits
@@ -307,6 +423,9 @@ def main() -> int:
     ap.add_argument("--weight-copies", type=int, default=4)
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-decode-mix", action="store_true")
+    ap.add_argument("--decode-layers", type=int, default=48)
+    ap.add_argument("--decode-steps", type=int, default=500)
     ap.add_argument("--cpu-sample", type=int, default=4096, help="tokens of the workload the CPU baseline runs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -346,6 +465,7 @@ def main() -> int:
             "M": M,
             "tokens_per_s": M / t_layer,
             "ms_per_step": t_layer * 1e3,
+            "call_us": layer_percentiles(pkg, torch, dev, weights, args.steps, args.variant),
             "n_active_experts": n_act,
             "layer_int8_tops": ops_layer / t_layer / 1e12,
             "layer_mfma_frac": ops_layer / t_layer / PEAK_INT8_OPS,
@@ -400,6 +520,8 @@ def main() -> int:
         out["weight_requant"] = time_weight_requant(pkg, torch, pkg.inputs.SHAPES[args.shape],
                                                     max(args.steps // 2, 1), max(args.warmup // 2, 1))
         out["mfma_ceiling"] = time_mfma_ceiling(pkg, torch)
+        if not args.no_decode_mix:
+            out["decode_mix"] = time_decode_mix(pkg, torch, args.shape, args.decode_layers, args.decode_steps)
     if not args.no_cpu:
         oracle = importlib.import_module("oracle.moe_i8_oracle")
         out["cpu_baseline"] = cpu_baseline(oracle, torch, base_headline, args.cpu_sample)
