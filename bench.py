@@ -372,6 +372,23 @@ def time_mfma_ceiling(pkg, torch) -> dict:
     return res
 
 
+def time_hbm_ceiling(torch) -> dict:
+    """What a plain device-to-device copy of 1 GiB sustains (bytes read plus bytes written per second):
+    the practical counterpart of the published HBM peak for the streaming kernels of the layer."""
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+    dst = torch.empty_like(src)
+    best = float("inf")
+    for _ in range(5):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        dst.copy_(src)
+        b.record()
+        torch.cuda.synchronize()
+        best = min(best, a.elapsed_time(b) * 1e-3)
+    return {"copy_GBps": 2 * n / best / 1e9, "frac_of_peak": 2 * n / best / PEAK_HBM_BPS, "unit": "GB/s"}
+
+
 def time_dense_mlp(pkg, torch, M: int, H: int, I: int, steps: int, warmup: int) -> dict:
     """The shared-expert / dense W8A8 gated MLP on the same GEMM kernels with one group."""
     g = torch.Generator(device="cuda:0").manual_seed(3)
@@ -520,6 +537,7 @@ def main() -> int:
         out["weight_requant"] = time_weight_requant(pkg, torch, pkg.inputs.SHAPES[args.shape],
                                                     max(args.steps // 2, 1), max(args.warmup // 2, 1))
         out["mfma_ceiling"] = time_mfma_ceiling(pkg, torch)
+        out["hbm_ceiling"] = time_hbm_ceiling(torch)
         if not args.no_decode_mix:
             out["decode_mix"] = time_decode_mix(pkg, torch, args.shape, args.decode_layers, args.decode_steps)
     if not args.no_cpu:
