@@ -202,6 +202,24 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
                          void* workspace, int64_t workspace_bytes, int variant, void* stream);
 
 /*
+ * moe_i8_fused_experts for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments and result as moe_i8_fused_experts without the workspace: the intermediate buffers
+ * live in a device array of MOE_I8_STATIC_SCRATCH_BYTES that is part of the library's code object
+ * (every GPU the library runs on holds its own copy until the process ends).  The call allocates and
+ * frees nothing.  A shape whose moe_i8_workspace_bytes() exceeds the array is rejected with
+ * MOE_I8_EWORKSPACE.  All calls on one GPU share the array: calls that overlap on one GPU (different
+ * streams or threads) race; calls ordered on one stream do not.  Nothing has to be cleared between
+ * calls: every region is written before it is read.
+ */
+#define MOE_I8_STATIC_SCRATCH_BYTES (32 << 20)
+int moe_i8_fused_experts_static(const void* hidden, const int8_t* w1, const int8_t* w2,
+                                const float* topk_weights, const int32_t* topk_ids,
+                                const float* w1_scale, const float* w2_scale, void* out, int64_t m,
+                                int top_k, int num_experts, int hidden_size, int inter, int block_size,
+                                int variant, void* stream);
+
+/*
  * Dense W8A8 layers (shared experts, dense first-k MLPs) on the same kernels with one group.
  *
  * moe_i8_scaled_int8_quant replaces vLLM `ops.scaled_int8_quant(x, scale=None)` (dynamic per-token

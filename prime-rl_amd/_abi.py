@@ -63,7 +63,12 @@ SIGNATURES = {
         c_int,
         [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, _P, c_int64, c_int, _P],
     ),
+    "moe_i8_fused_experts_static": (
+        c_int,
+        [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+    ),
 }
+STATIC_SCRATCH_BYTES = 32 << 20
 
 _lib = None
 

@@ -3,6 +3,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "../../include/moe_i8.h"
 #include "common.hpp"
 
@@ -566,6 +568,56 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
       return rc;
   }
   return moe_i8_sum(down, out, m, top_k, hidden_size, stream);
+}
+
+// ---- the entry point that allocates nothing ----
+// The workspace of the layer lives in a file-scope device array instead of caller memory.  The
+// array's name is only a host-side handle: the device address is asked from the runtime once per
+// device (each device holds its own copy at its own address) and that pointer is what the launches get.
+namespace {
+static __device__ __attribute__((used)) __align__(256) unsigned char scratch[MOE_I8_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void** out) {
+  int dev = -1;
+  const hipError_t derr = hipGetDevice(&dev);
+  if (derr != hipSuccess) return fail(MOE_I8_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(derr));
+  if (dev < 0 || dev >= kMaxDevices) return fail(MOE_I8_EUNSUPPORTED, "device index %d outside [0, %d)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    const hipError_t err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || !p)
+      return fail(MOE_I8_ELAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(err));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return MOE_I8_OK;
+}
+}  // namespace
+
+int moe_i8_fused_experts_static(const void* hidden, const int8_t* w1, const int8_t* w2,
+                                const float* topk_weights, const int32_t* topk_ids,
+                                const float* w1_scale, const float* w2_scale, void* out, int64_t m,
+                                int top_k, int num_experts, int hidden_size, int inter, int block_size,
+                                int variant, void* stream) {
+  if (m < 0) return fail(MOE_I8_EINVAL, "negative m");
+  if (m == 0) return MOE_I8_OK;
+  const int64_t need = moe_i8_workspace_bytes(m, top_k, num_experts, hidden_size, inter, block_size);
+  if (need < 0) return fail(MOE_I8_EINVAL, "bad layer shape");
+  if (need > (int64_t)MOE_I8_STATIC_SCRATCH_BYTES)
+    return fail(MOE_I8_EWORKSPACE,
+                "this call needs %lld bytes of scratch, the static array holds %lld: use moe_i8_fused_experts "
+                "with a caller-owned workspace",
+                (long long)need, (long long)MOE_I8_STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  // every region of the workspace is written by the call before it is read: nothing to clear
+  return moe_i8_fused_experts(hidden, w1, w2, topk_weights, topk_ids, w1_scale, w2_scale, out, m, top_k,
+                              num_experts, hidden_size, inter, block_size, ws, MOE_I8_STATIC_SCRATCH_BYTES, variant,
+                              stream);
 }
 
 // Workspace of the dense entry points (every region 256-byte aligned):
