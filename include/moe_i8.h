@@ -129,6 +129,9 @@ int moe_i8_quant_weights(const void* w, int dtype, int64_t rows, int64_t cols, i
  * trainer/models/layers/moe.py:146-148; activation trainer/models/layers/activations.py:29-34.
  * x_q int8 [M, H], a_scale fp32 [M], w1 int8 [E, 2I, H], w1_scale fp32 [E, 2I]
  * -> act bf16 [num_pairs, I], row t = pair t (token t / top_k).
+ * The routing may come from anywhere, with one requirement every router meets: the top_k experts
+ * of one token are distinct, so an expert holds at most num_pairs / top_k rows (the streaming
+ * family sizes its launch on that; rows beyond it would not be computed).
  */
 int moe_i8_gemm_gate_up_silu(const int8_t* x_q, const float* a_scale, const int8_t* w1,
                              const float* w1_scale, const int32_t* sorted_token_ids,
@@ -155,7 +158,9 @@ int moe_i8_gemm_down(const int8_t* h_q, const float* a_scale, const int8_t* w2,
  * The down GEMM with the second `per_token_quant_int8` folded in (streaming family only, inter <= 1024):
  * act bf16 [num_pairs, I] is quantised row by row inside the kernel with the arithmetic of
  * moe_i8_quant_rows, so the result equals moe_i8_quant_rows followed by moe_i8_gemm_down bit for bit.
- * moe_i8_fused_experts uses it whenever it picks the streaming family for the down GEMM.
+ * moe_i8_fused_experts uses it when it picks the streaming family for the down GEMM and experts hold
+ * at most three rows on average (num_pairs <= 3 * num_experts); with more rows the separate
+ * quantisation launch is the cheaper one, because every workgroup of a block repeats the quantisation.
  */
 int moe_i8_gemm_down_bf16(const void* act, const int8_t* w2, const float* w2_scale, const float* topk_weights,
                           const int32_t* sorted_token_ids, const int32_t* expert_ids,
@@ -193,7 +198,8 @@ int64_t moe_i8_workspace_bytes(int64_t m, int top_k, int num_experts, int hidden
  * synchronisation.  hidden bf16 [M, H]; out bf16 [M, H] (may alias hidden).
  * Every topk_id must lie in [0, num_experts): a pair with another id is skipped by the alignment and
  * the GEMMs, so its row of the intermediate buffer is never written and the combine would add
- * whatever the workspace holds there (expert-parallel maps are not part of this path).
+ * whatever the workspace holds there (expert-parallel maps are not part of this path).  The top_k
+ * ids of one token must be distinct (see moe_i8_gemm_gate_up_silu).
  */
 int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
                          const float* topk_weights, const int32_t* topk_ids,

@@ -24,6 +24,8 @@ from .api import (  # noqa: F401
     moe_sum,
     per_token_quant_int8,
     quantize_expert_weights,
+    load_quantized_expert_weights,
+    reserve_workspace,
     quantize_weights_per_channel,
     sorted_capacity,
     workspace_bytes,
@@ -37,6 +39,8 @@ __all__ = [
     "per_token_quant_int8",
     "quantize_weights_per_channel",
     "quantize_expert_weights",
+    "load_quantized_expert_weights",
+    "reserve_workspace",
     "moe_sum",
     "fused_topk",
     "grouped_topk",

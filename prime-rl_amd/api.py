@@ -12,6 +12,9 @@ eager fallback: without the built library, or off a GPU, these functions raise.
 
 from __future__ import annotations
 
+import threading
+from collections import OrderedDict
+
 import torch
 
 from . import _abi
@@ -23,6 +26,7 @@ __all__ = [
     "per_token_quant_int8",
     "quantize_weights_per_channel",
     "quantize_expert_weights",
+    "load_quantized_expert_weights",
     "moe_sum",
     "fused_topk",
     "grouped_topk",
@@ -36,13 +40,20 @@ __all__ = [
     "gemm_down_bf16",
     "gemm_acc_i32",
     "workspace_bytes",
+    "reserve_workspace",
     "sorted_capacity",
     "DEFAULT_BLOCK_SIZE_M",
 ]
 
 DEFAULT_BLOCK_SIZE_M = 64
 _VARIANTS = {"auto": _abi.GEMM_AUTO, "stream": _abi.GEMM_STREAM, "tile": _abi.GEMM_TILE, "narrow": _abi.GEMM_NARROW}
-_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+# Default workspaces, one per (device, stream) that has called without a caller-owned one: a small
+# LRU (a process has a handful of forward streams) guarded by a lock.  Entries are only ever created or
+# grown outside HIP graph capture, so a captured graph never holds a pointer that a later call frees:
+# a capture that finds no entry large enough raises instead of allocating.
+_MAX_CACHED_WORKSPACES = 16
+_workspaces: "OrderedDict[tuple[int, int], torch.Tensor]" = OrderedDict()
+_workspaces_lock = threading.Lock()
 
 
 def _ptr(t: torch.Tensor | None) -> int | None:
@@ -253,6 +264,67 @@ def quantize_expert_weights(
     return w13, s13, w2, s2
 
 
+_EXPERT_PARAM_SUFFIXES = ("w13_weight", "w13_weight_scale", "w2_weight", "w2_weight_scale")
+
+
+@torch.no_grad()
+def load_quantized_expert_weights(
+    params: dict,
+    prefix: str,
+    w1: torch.Tensor,
+    w3: torch.Tensor,
+    w2: torch.Tensor,
+    source_indices: torch.Tensor | None = None,
+) -> list[str]:
+    """Policy update of one int8 W8A8 MoE layer of a running engine: quantise the trainer's bf16
+    ``w1`` (gate) ``[E, I, H]``, ``w3`` (up) ``[E, I, H]`` and ``w2`` (down) ``[E, H, I]`` and write
+    ``w13_weight``, ``w13_weight_scale``, ``w2_weight``, ``w2_weight_scale`` of that layer in place, so
+    the addresses the engine (and any captured graph) holds stay valid.
+
+    The int8 counterpart of the reference's kernel-format weight transfer
+    (``src/prime_rl/inference/vllm/worker/weight_transfer.py:97-134``): ``params`` is
+    ``dict(model.named_parameters())``; the four tensors are looked up as ``{prefix}.{name}`` or, as the
+    pinned vLLM nests them, ``{prefix}.routed_experts.{name}`` (``weight_transfer.py:76-82``); a missing
+    name or a shape that does not match raises ``ValueError`` naming it, as the reference does, before
+    anything is written; ``source_indices`` selects the experts local to this worker from the trainer's
+    tensors the way ``tensor[source_indices]`` does there (``:120-125``).  Scales may be ``[E, N]`` or
+    ``[E, N, 1]``.  Returns the names written.
+    """
+    found, missing = {}, []
+    for suffix in _EXPERT_PARAM_SUFFIXES:
+        for name in (f"{prefix}.{suffix}", f"{prefix}.routed_experts.{suffix}"):
+            if name in params:
+                found[suffix] = (name, params[name])
+                break
+        else:
+            missing.append(f"{prefix}.{suffix}")
+    if missing:
+        raise ValueError(f"int8 expert weight update: {len(missing)} parameters not found in model: {missing}")
+    if source_indices is not None:
+        idx = source_indices.to(device=w1.device, dtype=torch.long)
+        w1, w3, w2 = w1[idx].contiguous(), w3[idx].contiguous(), w2[idx].contiguous()
+    if w1.dim() != 3 or w1.shape != w3.shape or w2.dim() != 3:
+        raise ValueError("w1 and w3 must be [E, I, H] and w2 [E, H, I]")
+    E, I, H = w1.shape
+    want = {"w13_weight": (E, 2 * I, H), "w13_weight_scale": (E, 2 * I), "w2_weight": (E, H, I),
+            "w2_weight_scale": (E, H)}
+    mismatches, views = [], {}
+    for suffix, (name, param) in found.items():
+        t = param.data if isinstance(param, torch.nn.Parameter) else param
+        shape = tuple(t.shape)
+        ok = shape == want[suffix] or (suffix.endswith("_scale") and shape == want[suffix] + (1,))
+        if tuple(w2.shape) != (E, H, I) or not ok:
+            mismatches.append(f"{name}: param={list(shape)} != received={list(want[suffix])}")
+            continue
+        views[suffix] = t.view(want[suffix]) if shape != want[suffix] else t
+    if mismatches:
+        raise ValueError(f"int8 expert weight update had {len(mismatches)} shape mismatches: {mismatches}")
+    quantize_expert_weights(
+        w1, w3, w2, out=(views["w13_weight"], views["w13_weight_scale"], views["w2_weight"], views["w2_weight_scale"])
+    )
+    return [found[suffix][0] for suffix in _EXPERT_PARAM_SUFFIXES]
+
+
 def moe_sum(input: torch.Tensor, output: torch.Tensor) -> None:
     """vLLM ``ops.moe_sum``: ``output[m] = sum_j input[m, j]`` for bf16 ``[M, k, H]`` → ``[M, H]``."""
     _require_gpu("input", input)
@@ -437,9 +509,17 @@ def _dense_weight(name: str, w: torch.Tensor, scale: torch.Tensor) -> torch.Tens
     return w
 
 
-def _dense_workspace(x: torch.Tensor, k: int, inter: int) -> torch.Tensor:
+def _dense_workspace(x: torch.Tensor, k: int, inter: int, workspace: torch.Tensor | None = None) -> torch.Tensor:
+    """Workspace of the dense entry points: the caller's (``moe_i8_dense_workspace_bytes`` bytes, needed
+    under graph capture unless one was cached earlier) or the cached per-(device, stream) one."""
     m = x.numel() // k
-    return _workspace(x.device, _stream(x), _abi.load().moe_i8_dense_workspace_bytes(m, k, inter))
+    need = _abi.load().moe_i8_dense_workspace_bytes(m, k, inter)
+    if workspace is None:
+        return _workspace(x.device, _stream(x), need)
+    _require_gpu("workspace", workspace)
+    if workspace.numel() * workspace.element_size() < need:
+        raise ValueError(f"workspace too small: need {need} bytes")
+    return workspace
 
 
 def apply_int8_linear(
@@ -452,6 +532,7 @@ def apply_int8_linear(
     bias: torch.Tensor | None = None,
     *,
     gemm_variant: str | int = "auto",
+    workspace: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """vLLM's dense W8A8 int8 linear (dynamic per-token symmetric activations, per-channel weights):
     ``scaled_int8_quant`` then ``cutlass_scaled_mm``; ``out = bf16((acc * a_scale) * w_scale)``.
@@ -469,10 +550,10 @@ def apply_int8_linear(
         raise ValueError(f"input has {input.shape[-1]} features, weight expects {k}")
     m = input.numel() // k
     out = torch.empty((*input.shape[:-1], n), dtype=torch.bfloat16, device=input.device)
-    ws = _dense_workspace(input, k, 0)
+    ws = _dense_workspace(input, k, 0, workspace)
     _abi.check(
         _abi.load().moe_i8_w8a8_linear(_ptr(input), _ptr(w), _ptr(weight_scale), _ptr(out), m, n, k, _ptr(ws),
-                                       ws.numel(), _variant(gemm_variant), _stream(input))
+                                       ws.numel() * ws.element_size(), _variant(gemm_variant), _stream(input))
     )
     return out
 
@@ -485,6 +566,7 @@ def w8a8_mlp(
     w2_scale: torch.Tensor,
     *,
     gemm_variant: str | int = "auto",
+    workspace: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Dense gated MLP ``down(silu(gate(x)) * up(x))`` in W8A8 (the shared expert the reference adds to the
     routed output, ``src/prime_rl/trainer/models/layers/moe.py:453-462``; ``FeedForward.forward``,
@@ -500,10 +582,10 @@ def w8a8_mlp(
         raise ValueError("expected x [*, H], w13 [2I, H], w2 [H, I]")
     m = x.numel() // h
     out = torch.empty_like(x)
-    ws = _dense_workspace(x, h, two_i // 2)
+    ws = _dense_workspace(x, h, two_i // 2, workspace)
     _abi.check(
         _abi.load().moe_i8_w8a8_mlp(_ptr(x), _ptr(w13), _ptr(w13_scale), _ptr(w2), _ptr(w2_scale), _ptr(out), m, h,
-                                    two_i // 2, _ptr(ws), ws.numel(), _variant(gemm_variant), _stream(x))
+                                    two_i // 2, _ptr(ws), ws.numel() * ws.element_size(), _variant(gemm_variant), _stream(x))
     )
     return out
 
@@ -635,13 +717,39 @@ def gemm_acc_i32(
 
 
 # --------------------------------------------------------------------------------------------- #
+def _capturing(device: torch.device) -> bool:
+    return bool(torch.cuda.is_available() and torch.cuda.is_current_stream_capturing())
+
+
 def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
+    with _workspaces_lock:
+        ws = _workspaces.get(key)
+        if ws is not None and ws.numel() >= nbytes:
+            _workspaces.move_to_end(key)
+            return ws
+        if _capturing(device):
+            raise RuntimeError(
+                f"this call needs a {nbytes}-byte workspace while the stream is being captured into a graph and "
+                "none of that size was allocated for it beforehand: pass workspace=, or call reserve_workspace() "
+                "(or run the largest batch once eagerly on this stream) before capturing"
+            )
         ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
-    return ws
+        _workspaces.move_to_end(key)
+        while len(_workspaces) > _MAX_CACHED_WORKSPACES:
+            _workspaces.popitem(last=False)
+        return ws
+
+
+def reserve_workspace(max_tokens: int, top_k: int, num_experts: int, hidden: int, inter: int, device=None,
+                      block_size_m: int = DEFAULT_BLOCK_SIZE_M) -> torch.Tensor:
+    """Allocate now (outside any graph capture) the default workspace that ``fused_experts`` calls on the
+    current stream of ``device`` use for up to ``max_tokens`` tokens of this layer shape, so that captured
+    calls find it.  The tensor stays cached for that (device, stream); it is also returned."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    return _workspace(device, stream, workspace_bytes(max_tokens, top_k, num_experts, hidden, inter, block_size_m))
 
 
 def fused_experts(
@@ -666,16 +774,22 @@ def fused_experts(
     block_size_m: int = DEFAULT_BLOCK_SIZE_M,
     gemm_variant: str | int = "auto",
     workspace: torch.Tensor | None = None,
+    out: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Drop-in for vLLM ``fused_experts`` on the INT8 W8A8 path (per-channel weight scales, dynamic
     per-token activation scales, SiLU-gated experts, routed weight applied after the experts).
 
     ``a1_scale`` / ``a2_scale`` are accepted for signature compatibility and ignored: with
-    per-token dynamic quantisation upstream recomputes them too.  The three keyword-only
-    arguments are extensions: the moe_align block size (64, as the baseline pins it), the GEMM
-    kernel family and an optional caller-owned workspace of ``workspace_bytes(...)`` bytes.
-    ``topk_ids`` must lie in ``[0, E)``: there is no expert map on this path, and a pair routed
-    nowhere would leave its row of the intermediate buffer unwritten.
+    per-token dynamic quantisation upstream recomputes them too.  The keyword-only arguments are
+    extensions: the moe_align block size (64, as the baseline pins it), the GEMM kernel family, an
+    optional caller-owned workspace of ``workspace_bytes(...)`` bytes and an optional bf16 ``[M, H]``
+    tensor to write the result into.  Without ``workspace`` a cached per-(device, stream) buffer is
+    used; it is never allocated or grown while the stream is being captured (see ``reserve_workspace``).
+
+    ``topk_ids`` must lie in ``[0, E)`` (there is no expert map on this path, and a pair routed
+    nowhere would leave its row of the intermediate buffer unwritten) and the ``k`` experts of one
+    token must be distinct, as every router produces them: the kernels size their work on an expert
+    holding at most one row per token.
     """
     if not use_int8_w8a8:
         raise NotImplementedError("this library implements only the use_int8_w8a8=True path")
@@ -719,7 +833,12 @@ def fused_experts(
     _require_gpu("topk_weights", topk_weights)
     block_size_m = _block_size(block_size_m)
     k = topk_ids.shape[1]
-    out = hidden_states if inplace else torch.empty_like(hidden_states)
+    if out is not None:
+        _require_gpu("out", out)
+        if out.shape != hidden_states.shape or out.dtype != torch.bfloat16:
+            raise ValueError("out must be bfloat16 with the shape of hidden_states")
+    else:
+        out = hidden_states if inplace else torch.empty_like(hidden_states)
     if M == 0:
         return out
     ids = _as_i32_ids(topk_ids)

@@ -8,37 +8,77 @@ variable because workers are spawned without config objects
 (``src/prime_rl/inference/vllm/worker/__init__.py:12-22``), and rebinds the name in every module
 that imported it with ``from ... import fused_experts`` (``patches.py:227-231``).
 
-Without vLLM installed ``register()`` is a no-op.  It cannot be exercised offline; it is kept thin
-and makes no parity claim of its own.
+Two surfaces are covered:
+
+* the flat ``fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, ..., use_int8_w8a8=True, ...)``
+  function: calls this library handles go to the HIP path, everything else (another quantisation
+  mode, an expert map, a keyword this library does not know, a shape it rejects) falls through to
+  the original;
+* the modular-kernel surface the pinned vLLM selects kernels through (``FusedMoE`` is a factory
+  returning a ``MoERunner``, reference ``src/prime_rl/inference/vllm/worker/weight_transfer.py:76-82``;
+  the choice of experts implementation goes through ``FusedMoEConfig``, ``patches.py:740-757``):
+  ``Int8W8A8HipExperts`` has the ``apply(output, hidden_states, w1, w2, topk_weights, topk_ids, ...)``
+  shape of an experts implementation and forwards to the same C-ABI driver.
+
+Nothing here allocates under HIP graph capture: a call made while the stream is capturing uses a
+workspace that was allocated beforehand for that (device, stream) by ``reserve_workspace`` or by an
+earlier eager call of at least the same size, and raises otherwise.
+
+Without vLLM installed ``register()`` is a no-op.  vLLM itself cannot be run offline; the
+rebinding, marker and fall-through logic is exercised against a stand-in module tree in the CPU tests.
 """
 
 from __future__ import annotations
 
 import importlib
+import inspect
 import os
 import sys
 
 ENV_FLAG = "PRIME_MOE_I8_HIP"
 _MARK = "_prime_moe_i8_hip_patched"
+FUSED_MOE_MODULE = "vllm.model_executor.layers.fused_moe.fused_moe"
+# keywords of vLLM's flat signature that select another code path when truthy: the HIP path is only
+# taken when all of them are absent or falsy
+_OTHER_MODE_FLAGS = (
+    "use_fp8_w8a8", "use_int8_w8a16", "use_int4_w4a16", "use_mxfp4_w4a4", "use_nvfp4_w4a4", "ocp_mx_scheme",
+    "w1_zp", "w2_zp", "w1_bias", "w2_bias", "allow_deep_gemm", "allow_cutlass_block_scaled_grouped_gemm",
+    "apply_router_weight_on_input", "expert_map", "block_shape",
+)
 
 
-def _wrap(original):
-    from .api import fused_experts as hip_fused_experts
+def _accepted_keywords(fn) -> frozenset:
+    return frozenset(
+        name for name, p in inspect.signature(fn).parameters.items()
+        if p.kind in (inspect.Parameter.POSITIONAL_OR_KEYWORD, inspect.Parameter.KEYWORD_ONLY)
+    )
+
+
+def _handles(hidden_states, kwargs, accepted) -> bool:
+    if not kwargs.get("use_int8_w8a8", False) or not kwargs.get("per_channel_quant", False):
+        return False
+    if kwargs.get("activation", "silu") != "silu":
+        return False
+    if any(kwargs.get(flag) for flag in _OTHER_MODE_FLAGS):
+        return False
+    # a keyword this library has never heard of may change the meaning of the call
+    if any(k not in accepted and k not in _OTHER_MODE_FLAGS and v not in (None, False) for k, v in kwargs.items()):
+        return False
+    return bool(getattr(hidden_states, "is_cuda", False)) and str(getattr(hidden_states, "dtype", "")) == "torch.bfloat16"
+
+
+def _wrap(original, hip_fused_experts=None):
+    if hip_fused_experts is None:
+        from .api import fused_experts as hip_fused_experts
+    accepted = _accepted_keywords(hip_fused_experts)
 
     def fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, *args, **kwargs):
-        use_hip = (
-            kwargs.get("use_int8_w8a8", False)
-            and kwargs.get("per_channel_quant", False)
-            and kwargs.get("expert_map") is None
-            and kwargs.get("block_shape") is None
-            and kwargs.get("activation", "silu") == "silu"
-            and not kwargs.get("apply_router_weight_on_input", False)
-            and not args
-            and hidden_states.is_cuda
-            and str(hidden_states.dtype) == "torch.bfloat16"
-        )
-        if use_hip:
-            return hip_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, **kwargs)
+        if not args and _handles(hidden_states, kwargs, accepted):
+            forwarded = {k: v for k, v in kwargs.items() if k in accepted}
+            try:
+                return hip_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, **forwarded)
+            except (NotImplementedError, TypeError):
+                pass  # a mode or shape this library rejects: the original handles it
         return original(hidden_states, w1, w2, topk_weights, topk_ids, *args, **kwargs)
 
     setattr(fused_experts, _MARK, True)
@@ -51,7 +91,7 @@ def register() -> bool:
     if os.environ.get(ENV_FLAG, "0") != "1":
         return False
     try:
-        fm = importlib.import_module("vllm.model_executor.layers.fused_moe.fused_moe")
+        fm = importlib.import_module(FUSED_MOE_MODULE)
     except ImportError:
         return False
     original = getattr(fm, "fused_experts", None)
@@ -65,3 +105,54 @@ def register() -> bool:
         if getattr(mod, "fused_experts", None) is original:
             mod.fused_experts = patched
     return True
+
+
+def reserve_workspace(max_tokens: int, top_k: int, num_experts: int, hidden: int, inter: int, device=None,
+                      block_size_m: int = 64):
+    """Allocate, before any graph capture, the workspace calls on the current stream of `device` will use
+    for batches of up to `max_tokens` tokens.  Returns the tensor (the cache keeps it alive)."""
+    from . import api
+
+    return api.reserve_workspace(max_tokens, top_k, num_experts, hidden, inter, device=device,
+                                 block_size_m=block_size_m)
+
+
+class Int8W8A8HipExperts:
+    """Experts implementation with the ``apply`` shape of vLLM's modular MoE kernels
+    (``TritonExperts.apply(output, hidden_states, w1, w2, topk_weights, topk_ids, activation,
+    global_num_experts, expert_map, a1q_scale, a2_scale, workspace13, workspace2, ...)``) for channel-wise
+    int8 weights with dynamic per-token activation scales (what ``int8_w8a8_moe_quant_config(w1_scale,
+    w2_scale, per_act_token_quant=True)`` describes).  ``apply`` writes the layer's result into ``output``.
+
+    The activation quantisation runs inside the library, so ``hidden_states`` is the bf16 input and an
+    ``a1q_scale`` handed over by a prepare step that has already quantised is refused (that pairing
+    would quantise twice).  vLLM's two workspace tensors are not used: the library's own workspace
+    holds its intermediates.
+    """
+
+    def __init__(self, w1_scale, w2_scale, block_size_m: int = 64, gemm_variant: str = "auto"):
+        self.w1_scale = w1_scale
+        self.w2_scale = w2_scale
+        self.block_size_m = block_size_m
+        self.gemm_variant = gemm_variant
+
+    def supports_expert_map(self) -> bool:
+        return False
+
+    def supports_chunking(self) -> bool:
+        return True
+
+    def apply(self, output, hidden_states, w1, w2, topk_weights, topk_ids, activation="silu",
+              global_num_experts=-1, expert_map=None, a1q_scale=None, a2_scale=None, workspace13=None,
+              workspace2=None, expert_tokens_meta=None, apply_router_weight_on_input=False, **_unused):
+        from . import api
+
+        if a1q_scale is not None:
+            raise NotImplementedError("hidden_states must be the unquantised bf16 input (a1q_scale is None)")
+        result = api.fused_experts(
+            hidden_states, w1, w2, topk_weights, topk_ids, inplace=False, activation=activation,
+            apply_router_weight_on_input=apply_router_weight_on_input, use_int8_w8a8=True, per_channel_quant=True,
+            global_num_experts=global_num_experts, expert_map=expert_map, w1_scale=self.w1_scale,
+            w2_scale=self.w2_scale, block_size_m=self.block_size_m, gemm_variant=self.gemm_variant, out=output,
+        )
+        return result

@@ -165,3 +165,38 @@ def test_gemm_is_deterministic(pra, oracle, variant):
     first = _skip_if_unsupported(pra, lambda: pra.gemm_gate_up_silu(*args, variant))
     for _ in range(3):
         assert torch.equal(first, pra.gemm_gate_up_silu(*args, variant))
+
+
+# The GEMM shapes of the GLM-4.5-Air and DeepSeek-V3 layers (many channel tiles, long reductions):
+# int32 accumulators of every family that accepts the shape, all rows against each other on the
+# device and a few hundred sampled rows against the oracle's exact integer product.
+REAL_GEMM_SHAPES = [
+    # E, N, K, rows per expert (about), row_div
+    (8, 2 * 1408, 4096, 300, 8),   # GLM-4.5-Air gate_up
+    (8, 4096, 1408, 300, 1),       # GLM-4.5-Air down
+    (4, 4096, 7168, 400, 8),       # DeepSeek-V3 gate_up
+    (4, 7168, 2048, 400, 1),       # DeepSeek-V3 down
+]
+
+
+@pytest.mark.parametrize("E,N,K,rows,row_div", REAL_GEMM_SHAPES, ids=lambda v: str(v))
+def test_int32_accumulators_at_real_gemm_shapes(pra, oracle, E, N, K, rows, row_div):
+    g = torch.Generator().manual_seed(N + K)
+    P = E * rows
+    M = (P + row_div - 1) // row_div
+    a = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (E, N, K), generator=g, dtype=torch.int8)
+    ids = torch.randint(0, E, (P, 1), generator=g, dtype=torch.int32)
+    s, e, npp = pra.moe_align_block_size(ids.to(DEV), 64, E)
+    a_d, w_d = a.to(DEV), w.to(DEV)
+    got = {}
+    for variant in VARIANTS:
+        acc = _none_if_unsupported(pra, lambda: pra.gemm_acc_i32(a_d, w_d, s, e, npp, row_div, 64, P, variant))
+        if acc is not None:
+            got[variant] = acc
+    assert "stream" in got and len(got) >= 2, sorted(got)
+    for variant, acc in got.items():
+        assert torch.equal(acc, got["stream"]), variant
+    sel = torch.randperm(P, generator=g)[:256]
+    want = oracle.grouped_int_gemm(a[sel // row_div], w, ids[sel], 1)
+    assert torch.equal(got["stream"][sel.to(DEV)].cpu(), want)

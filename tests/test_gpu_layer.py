@@ -197,3 +197,65 @@ def test_small_batch_layer_equals_the_chain_of_its_stages(pra, E, k, H, I, M, B)
             torch.cuda.synchronize()
             same = bool(torch.equal(out, want))
             assert same, (routing, fill, int((out != want).sum()))
+
+
+# Whole-output checks at full size.  The sampled-token comparison above sees 6 rows; a tile
+# scheduler that dropped or duplicated a tile elsewhere would leave finite stale rows there.  The
+# streaming family uses none of the tiled families' scheduling code (one workgroup per block and
+# channel group, no persistent loop, no tile list), so bit-equality of the complete outputs of two
+# families over every row is a check of all of them.  The families share one SiLU definition and
+# the same integer accumulators, so the layer output is bit-identical by construction.
+FULL_SIZE = [
+    ("qwen3-30b-a3b", 8192), ("glm-4.5-air", 4096), ("deepseek-v3", 2048), ("deepseek-v3", 16384),
+]
+
+
+@pytest.mark.parametrize("shape_name,M", FULL_SIZE)
+def test_full_size_whole_output_equal_across_families(pra, shape_name, M):
+    im = inputs_mod()
+    inp = im.make_inputs(shape_name, M, seed=M + 7, device=DEV, weights_on_device=True)
+    auto = _run(pra, inp, gemm_variant="auto")
+    stream = _run(pra, inp, gemm_variant="stream")
+    assert bool(torch.isfinite(auto.float()).all())
+    differing = int((auto != stream).sum())
+    assert differing == 0, f"{differing} of {auto.numel()} elements differ between the families"
+    # and stage by stage on the device: the down GEMM of the tiled family against the streaming one
+    P = M * inp.topk_ids.shape[1]
+    x_q, a1 = pra.per_token_quant_int8(inp.hidden_states)
+    E = inp.w1.shape[0]
+    s, e, npp = pra.moe_align_block_size(inp.topk_ids, 64, E)
+    act = pra.gemm_gate_up_silu(x_q, a1, inp.w1, inp.w1_scale, s, e, npp, inp.topk_ids.shape[1], 64, P, "stream")
+    h_q, a2 = pra.per_token_quant_int8(act)
+    d_auto = pra.gemm_down(h_q, a2, inp.w2, inp.w2_scale, inp.topk_weights, s, e, npp, 64, "auto")
+    d_stream = pra.gemm_down(h_q, a2, inp.w2, inp.w2_scale, inp.topk_weights, s, e, npp, 64, "stream")
+    assert torch.equal(d_auto, d_stream)
+
+
+def test_capture_never_allocates_the_default_workspace(pra):
+    """Under HIP graph capture the default workspace is never created or grown: a capture that finds
+    none raises, one that finds a reserved buffer replays correctly after a larger eager call."""
+    im = inputs_mod()
+    inp = im.make_inputs("qwen3-30b-a3b", 32, seed=5).to(DEV)
+    big = im.make_inputs("qwen3-30b-a3b", 256, seed=6).to(DEV)
+    eager = _run(pra, inp)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with pytest.raises(RuntimeError, match="reserve_workspace"):
+            with torch.cuda.graph(graph, stream=stream):
+                pra.fused_experts(*inp.fused_experts_args(), **inp.fused_experts_kwargs())
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        shape = im.SHAPES["qwen3-30b-a3b"]
+        pra.reserve_workspace(256, shape.k, shape.E_total, shape.H, shape.I)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            out = pra.fused_experts(*inp.fused_experts_args(), **inp.fused_experts_kwargs())
+        for _ in range(3):
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager)
+            # eager work at the reserved size on the same stream between replays: same buffer, no regrowth
+            pra.fused_experts(*big.fused_experts_args(), **big.fused_experts_kwargs())
+            torch.cuda.synchronize()

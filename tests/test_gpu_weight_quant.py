@@ -114,3 +114,56 @@ def test_argument_errors(pra):
         pra.quantize_weights_per_channel(w.cpu())
     with pytest.raises(ValueError):
         pra.quantize_expert_weights(w.view(1, 4, 16), w.view(1, 4, 16), w.view(1, 4, 16))
+
+
+def test_policy_update_hook_writes_layer_parameters_in_place(pra, oracle):
+    """``load_quantized_expert_weights`` (the int8 counterpart of the reference's in-place
+    ``param.copy_`` loop, src/prime_rl/inference/vllm/worker/weight_transfer.py:97-134): the four
+    parameters of the named layer are rewritten at their addresses, the layer's output afterwards is
+    the oracle's on the re-quantised weights, another layer in the same dict is untouched, and a
+    missing name or a wrong shape raises before anything is written."""
+    im = inputs_mod()
+    shape = im.SHAPES["toy"]
+    E, I, H = shape.E_total, shape.I, shape.H
+    old = pra.quantize_expert_weights(*[t.to(DEV) for t in _weights(E, I, H, seed=20, spread=False)])
+    other = pra.quantize_expert_weights(*[t.to(DEV) for t in _weights(E, I, H, seed=21, spread=False)])
+    names = ("w13_weight", "w13_weight_scale", "w2_weight", "w2_weight_scale")
+    params = {}
+    for layer, tensors, nested in (("model.layers.0.mlp.experts", old, ".routed_experts"),
+                                   ("model.layers.1.mlp.experts", other, "")):
+        for name, t in zip(names, tensors):
+            if name.endswith("_scale"):
+                t = t.unsqueeze(-1).contiguous()  # the engine keeps [E, N, 1]
+            params[f"{layer}{nested}.{name}"] = torch.nn.Parameter(t, requires_grad=False)
+    ptrs = {k: v.data_ptr() for k, v in params.items()}
+    before_other = {k: v.detach().clone() for k, v in params.items() if ".layers.1." in k}
+    new = _weights(E, I, H, seed=22, spread=False)
+    written = pra.load_quantized_expert_weights(params, "model.layers.0.mlp.experts", *[t.to(DEV) for t in new])
+    assert written == [f"model.layers.0.mlp.experts.routed_experts.{n}" for n in names]
+    assert {k: v.data_ptr() for k, v in params.items()} == ptrs
+    for k, v in before_other.items():
+        assert torch.equal(params[k], v)
+    want = oracle.quantize_expert_weights(*new)
+    got = [params[f"model.layers.0.mlp.experts.routed_experts.{n}"] for n in names]
+    assert torch.equal(got[0].cpu(), want[0]) and torch.equal(got[1].cpu().squeeze(-1), want[1])
+    assert torch.equal(got[2].cpu(), want[2]) and torch.equal(got[3].cpu().squeeze(-1), want[3])
+    x = torch.randn(40, H, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16)
+    tw, ids = im.route(shape, 40, torch.Generator().manual_seed(6))
+    out = pra.fused_experts(x.to(DEV), got[0], got[2], tw.to(DEV), ids.to(DEV), use_int8_w8a8=True,
+                            per_channel_quant=True, w1_scale=got[1], w2_scale=got[3])
+    ref = oracle.fused_experts(x, want[0], want[2], tw, ids, want[1], want[3])
+    assert rel_err(out.cpu(), ref) < 1e-2
+    # a worker that holds a subset of the experts takes its rows of the trainer's tensors
+    sub = torch.tensor([5, 1, 6], device=DEV)
+    small = {f"l.{n}": torch.nn.Parameter(t[:3].clone(), requires_grad=False) for n, t in zip(names, old)}
+    pra.load_quantized_expert_weights(small, "l", *[t.to(DEV) for t in new], source_indices=sub)
+    assert torch.equal(small["l.w13_weight"].cpu(), want[0][[5, 1, 6]])
+    assert torch.equal(small["l.w2_weight_scale"].cpu(), want[3][[5, 1, 6]])
+    # errors come before any write
+    snapshot = got[0].detach().clone()
+    with pytest.raises(ValueError, match="not found in model"):
+        pra.load_quantized_expert_weights(params, "model.layers.7.mlp.experts", *[t.to(DEV) for t in new])
+    with pytest.raises(ValueError, match="shape mismatches"):
+        pra.load_quantized_expert_weights(params, "model.layers.0.mlp.experts",
+                                          *[t[:4].to(DEV) for t in new])
+    assert torch.equal(got[0], snapshot)

@@ -1,0 +1,153 @@
+"""The vLLM plugin shim against a stand-in ``vllm`` module tree (vLLM itself is not installable here):
+environment gate, idempotence through the marker attribute (the reference's pattern,
+``src/prime_rl/inference/patches.py:57-58``), rebinding in modules that imported the name
+(``patches.py:227-231``), fall-through for calls this library does not handle, keyword filtering, and
+the ``apply``-shaped adapter.  No GPU: the HIP entry is replaced by a recorder."""
+
+import sys
+import types
+
+import pytest
+import torch
+
+
+class _FakeCudaBf16:
+    """Enough of a tensor for the dispatch decision."""
+    is_cuda = True
+    dtype = torch.bfloat16
+
+
+def _install_fake_vllm(monkeypatch):
+    calls = []
+
+    def original_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, *args, **kwargs):
+        calls.append(("original", kwargs))
+        return "original"
+
+    names = ["vllm", "vllm.model_executor", "vllm.model_executor.layers", "vllm.model_executor.layers.fused_moe",
+             "vllm.model_executor.layers.fused_moe.fused_moe", "vllm.model_executor.layers.fused_moe.layer",
+             "vllm.model_executor.layers.quantization"]
+    mods = {n: types.ModuleType(n) for n in names}
+    mods["vllm.model_executor.layers.fused_moe.fused_moe"].fused_experts = original_fused_experts
+    # two modules that did `from ...fused_moe import fused_experts` at import time, one that did not
+    mods["vllm.model_executor.layers.fused_moe"].fused_experts = original_fused_experts
+    mods["vllm.model_executor.layers.fused_moe.layer"].fused_experts = original_fused_experts
+    mods["vllm.model_executor.layers.quantization"].fused_experts = lambda *a, **k: "unrelated"
+    for n, m in mods.items():
+        monkeypatch.setitem(sys.modules, n, m)
+    return mods, original_fused_experts, calls
+
+
+@pytest.fixture
+def plugin(pra, monkeypatch):
+    hip_calls = []
+
+    def hip_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, inplace=False, activation="silu",
+                          apply_router_weight_on_input=False, use_int8_w8a8=False, per_channel_quant=False,
+                          global_num_experts=-1, expert_map=None, w1_scale=None, w2_scale=None, a1_scale=None,
+                          a2_scale=None, block_shape=None, *, workspace=None):
+        hip_calls.append(dict(use_int8_w8a8=use_int8_w8a8, w1_scale=w1_scale, global_num_experts=global_num_experts))
+        if w1_scale == "unsupported-shape":
+            raise NotImplementedError("shape")
+        return "hip"
+
+    monkeypatch.setattr(pra.api, "fused_experts", hip_fused_experts)
+    return pra.vllm_plugin, hip_calls
+
+
+def test_register_is_gated_by_the_environment(plugin, monkeypatch):
+    vp, _ = plugin
+    mods, original, _ = _install_fake_vllm(monkeypatch)
+    monkeypatch.delenv(vp.ENV_FLAG, raising=False)
+    assert vp.register() is False
+    monkeypatch.setenv(vp.ENV_FLAG, "0")
+    assert vp.register() is False
+    assert mods[vp.FUSED_MOE_MODULE].fused_experts is original
+
+
+def test_register_rebinds_every_importer_once(plugin, monkeypatch):
+    vp, _ = plugin
+    mods, original, _ = _install_fake_vllm(monkeypatch)
+    monkeypatch.setenv(vp.ENV_FLAG, "1")
+    assert vp.register() is True
+    patched = mods[vp.FUSED_MOE_MODULE].fused_experts
+    assert patched is not original and getattr(patched, vp._MARK) is True and patched.__wrapped__ is original
+    assert mods["vllm.model_executor.layers.fused_moe"].fused_experts is patched
+    assert mods["vllm.model_executor.layers.fused_moe.layer"].fused_experts is patched
+    # a different function that happens to carry the same name is left alone
+    assert mods["vllm.model_executor.layers.quantization"].fused_experts() == "unrelated"
+    # second call: the marker makes it a no-op, nothing is wrapped twice
+    assert vp.register() is False
+    assert mods[vp.FUSED_MOE_MODULE].fused_experts is patched
+
+
+def test_dispatch_and_fall_through(plugin, monkeypatch):
+    vp, hip_calls = plugin
+    mods, _, calls = _install_fake_vllm(monkeypatch)
+    monkeypatch.setenv(vp.ENV_FLAG, "1")
+    vp.register()
+    fe = mods[vp.FUSED_MOE_MODULE].fused_experts
+    x = _FakeCudaBf16()
+    int8 = dict(use_int8_w8a8=True, per_channel_quant=True, w1_scale="s1", w2_scale="s2")
+    # the int8 W8A8 call, with the other mode flags a flat-signature caller passes along
+    assert fe(x, 1, 2, 3, 4, **int8, use_fp8_w8a8=False, use_int8_w8a16=False, w1_zp=None, allow_deep_gemm=False,
+              global_num_experts=8) == "hip"
+    assert hip_calls[-1] == dict(use_int8_w8a8=True, w1_scale="s1", global_num_experts=8)
+    # everything else goes to the original, arguments untouched
+    for other in (dict(use_fp8_w8a8=True), dict(expert_map="map"), dict(block_shape=[128, 128]),
+                  dict(apply_router_weight_on_input=True), dict(activation="gelu"), dict(per_channel_quant=False),
+                  dict(some_future_flag=True)):
+        n = len(hip_calls)
+        assert fe(x, 1, 2, 3, 4, **{**int8, **other}) == "original"
+        assert len(hip_calls) == n and calls[-1][1] == {**int8, **other}
+    assert fe(x, 1, 2, 3, 4, use_int8_w8a8=False) == "original"
+    cpu = types.SimpleNamespace(is_cuda=False, dtype=torch.bfloat16)
+    assert fe(cpu, 1, 2, 3, 4, **int8) == "original"
+    fp16 = types.SimpleNamespace(is_cuda=True, dtype=torch.float16)
+    assert fe(fp16, 1, 2, 3, 4, **int8) == "original"
+    # positional extras (an older signature) are not guessed at
+    assert fe(x, 1, 2, 3, 4, True, **int8) == "original"
+    # a shape the library rejects falls through instead of failing the forward pass
+    assert fe(x, 1, 2, 3, 4, **{**int8, "w1_scale": "unsupported-shape"}) == "original"
+
+
+def test_apply_adapter_forwards_to_the_flat_entry(pra, monkeypatch):
+    seen = {}
+
+    def fake(hidden_states, w1, w2, topk_weights, topk_ids, **kw):
+        seen.update(kw, hidden_states=hidden_states)
+        return kw["out"]
+
+    monkeypatch.setattr(pra.api, "fused_experts", fake)
+    experts = pra.vllm_plugin.Int8W8A8HipExperts("s1", "s2", block_size_m=64)
+    out = object()
+    assert experts.apply(out, "x", "w1", "w2", "tw", "ids", activation="silu", global_num_experts=128,
+                         expert_map=None, a1q_scale=None, a2_scale=None, workspace13="ws13", workspace2="ws2",
+                         expert_tokens_meta=None, apply_router_weight_on_input=False) is out
+    assert seen["use_int8_w8a8"] is True and seen["per_channel_quant"] is True and seen["out"] is out
+    assert seen["w1_scale"] == "s1" and seen["w2_scale"] == "s2" and seen["global_num_experts"] == 128
+    assert not experts.supports_expert_map()
+    with pytest.raises(NotImplementedError, match="a1q_scale"):
+        experts.apply(out, "x_q", "w1", "w2", "tw", "ids", a1q_scale="already quantised")
+
+
+def test_default_workspace_cache_is_bounded(pra, monkeypatch):
+    api = pra.api
+    monkeypatch.setattr(api, "_workspaces", type(api._workspaces)())
+    made = []
+    real_empty = torch.empty
+
+    def fake_empty(shape, dtype=None, device=None):
+        t = real_empty(shape, dtype=dtype)  # CPU stand-in
+        made.append(t)
+        return t
+
+    monkeypatch.setattr(api.torch, "empty", fake_empty)
+    dev = torch.device("cuda", 0)
+    for stream in range(api._MAX_CACHED_WORKSPACES + 5):
+        api._workspace(dev, stream, 1024)
+    assert len(api._workspaces) == api._MAX_CACHED_WORKSPACES
+    # the most recent streams stay; a hit does not allocate
+    n = len(made)
+    assert api._workspace(dev, api._MAX_CACHED_WORKSPACES + 4, 512) is made[-1]
+    assert len(made) == n
