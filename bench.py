@@ -34,16 +34,18 @@ SWEEP_M = (16, 128, 512, 1024, 8192)
 
 
 def _profile_traffic(kernel: str, M: int):
-    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE, each scaled by
-    what the counter reads for a plain copy of known size), when a summary for this kernel and batch
-    size has been recorded under profiles/; otherwise None."""
-    path = ROOT / "profiles" / "hbm_traffic_gate_up.txt"
+    """HBM bytes per launch from the rocprofv3 --pmc summary committed under profiles/ (FETCH_SIZE and
+    WRITE_SIZE, each scaled by what the counter reads for a plain copy of known size), when one has
+    been recorded for this kernel and batch size; otherwise None.  A hardware counter cannot be read from
+    inside this process, so the figure is a recorded one and says where it was recorded."""
+    name = "profiles/hbm_traffic_gate_up.txt"
+    path = ROOT / name
     if not path.exists():
         return None
     for line in path.read_text().splitlines():
         f = line.split()
         if len(f) == 7 and f[0] == "traffic" and f[1] == kernel and f[2] == f"M={M}":
-            return (float(f[3]) * float(f[5]) + float(f[4]) * float(f[6])) * 1024.0
+            return {"bytes": (float(f[3]) * float(f[5]) + float(f[4]) * float(f[6])) * 1024.0, "source": name}
     return None
 
 
@@ -350,25 +352,63 @@ def time_mfma_ceiling(pkg, torch) -> dict:
     """What the device sustains on a register-only int8 MFMA loop (no memory traffic at all) with constant
     and with pseudo-random operand bits: the board's power limit lowers the clock as the operand bits
     toggle, so the second figure, not the published peak, is the ceiling of any int8 GEMM on real data
-    here.  One launch of a few milliseconds on one workgroup per compute unit, best of four."""
-    lib, abi = pkg._abi.load(), pkg._abi
-    wgs = torch.cuda.get_device_properties(0).multi_processor_count
-    iters = 20000
-    sink = torch.empty(wgs * 512, dtype=torch.int32, device="cuda:0")
-    stream = torch.cuda.current_stream().cuda_stream
-    ops = lib.moe_i8_probe_mfma_ops(wgs, iters)
-    res = {"unit": "TFLOP/s", "note": "int8 TOP/s, v_mfma_i32_32x32x32_i8 from registers on every compute unit"}
-    for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
-        best = float("inf")
-        for _ in range(4):
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            abi.check(lib.moe_i8_probe_mfma(rnd, wgs, iters, sink.data_ptr(), sink.numel() * 4, stream))
-            b.record()
-            torch.cuda.synchronize()
-            best = min(best, a.elapsed_time(b) * 1e-3)
-        res[name] = ops / best / 1e12
-        res[name + "_frac_of_peak"] = ops / best / PEAK_INT8_OPS
+    here.  One launch of a few milliseconds on one workgroup per compute unit, best of four.  Next to it,
+    as a datum that owes nothing to this repository: the vendor library's dense int8 GEMM (torch._int_mm)
+    on the problem the gate_up GEMM of the headline point would be without experts, on the same kind of
+    random data."""
+    import ctypes
+
+    res = {"unit": "TOP/s", "note": "int8 operations per second, v_mfma_i32_32x32x32_i8 from registers on every "
+                                    "compute unit"}
+    path = pkg._abi.PROBE_LIB_PATH
+    if path.exists():
+        lib = ctypes.CDLL(str(path))
+        lib.moe_i8_probe_mfma_ops.restype = ctypes.c_double
+        lib.moe_i8_probe_mfma_ops.argtypes = [ctypes.c_int, ctypes.c_int]
+        lib.moe_i8_probe_mfma.restype = ctypes.c_int
+        lib.moe_i8_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_longlong,
+                                          ctypes.c_void_p]
+        wgs = torch.cuda.get_device_properties(0).multi_processor_count
+        iters = 20000
+        sink = torch.empty(wgs * 512, dtype=torch.int32, device="cuda:0")
+        stream = torch.cuda.current_stream().cuda_stream
+        ops = lib.moe_i8_probe_mfma_ops(wgs, iters)
+        for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
+            best = float("inf")
+            for _ in range(4):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                rc = lib.moe_i8_probe_mfma(rnd, wgs, iters, sink.data_ptr(), sink.numel() * 4, stream)
+                b.record()
+                torch.cuda.synchronize()
+                if rc != 0:
+                    raise RuntimeError(f"MFMA probe launch failed with HIP error {rc}")
+                best = min(best, a.elapsed_time(b) * 1e-3)
+            res[name] = ops / best / 1e12
+            res[name + "_frac_of_peak"] = ops / best / PEAK_INT8_OPS
+    else:
+        res["constant_operands"] = res["random_operands"] = None
+    m, k, n = 65536, 2048, 1536
+    try:
+        g = torch.Generator(device="cuda:0").manual_seed(7)
+        a_ = torch.randint(-127, 128, (m, k), generator=g, dtype=torch.int8, device="cuda:0")
+        b_ = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8, device="cuda:0")
+        for _ in range(3):
+            torch._int_mm(a_, b_.t())
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(10)]
+        torch.cuda.synchronize()
+        for e0, e1 in pairs:
+            e0.record()
+            torch._int_mm(a_, b_.t())
+            e1.record()
+        torch.cuda.synchronize()
+        t = sum(e0.elapsed_time(e1) for e0, e1 in pairs) / len(pairs) * 1e-3
+        res["library_int_mm"] = {"m": m, "k": k, "n": n, "us": t * 1e6, "int8_tops": 2.0 * m * k * n / t / 1e12,
+                                 "frac_of_peak": 2.0 * m * k * n / t / PEAK_INT8_OPS,
+                                 "note": "torch._int_mm (vendor library), dense, no scale epilogue, no SiLU"}
+    except Exception as exc:  # the datum is optional: a build of torch without the routine must not fail the bench
+        res["library_int_mm"] = None
+        res["library_int_mm_error"] = repr(exc)[:200]
     return res
 
 
@@ -409,6 +449,63 @@ def time_dense_mlp(pkg, torch, M: int, H: int, I: int, steps: int, warmup: int) 
     return {"M": M, "H": H, "I": I, "us": t * 1e6, "int8_tops": ops / t / 1e12, "mfma_frac": ops / t / PEAK_INT8_OPS}
 
 
+OTHER_SHAPES = (
+    ("glm-4.5-air", (32, 512, 4096)),  # Zipf-skewed routing, one always-on shared expert as expert id E
+    ("deepseek-v3", (8, 64, 2048, 16384)),  # grouped top-k, all 256 experts on the one GPU
+)
+
+
+def time_other_shape(pkg, torch, oracle, shape_name: str, M: int, steps: int, warmup: int, cpu: bool) -> dict:
+    """One layer-level line for a shape that is a parity case, not the headline: layer time, the
+    algorithmic HBM / MFMA fractions of the sampled routing, the padded-row ratio of moe_align, and
+    (for the small batches) the CPU checker's time on the experts this batch touches.  The weights of
+    these shapes (2-11 GB) are far larger than the 256 MB last-level cache, so one copy is enough."""
+    shape = pkg.inputs.SHAPES[shape_name]
+    inp = pkg.inputs.make_inputs(shape, M, seed=M + 3, device="cuda:0", weights_on_device=True)
+
+    def step():
+        return pkg.fused_experts(*inp.fused_experts_args(), **inp.fused_experts_kwargs())
+
+    for _ in range(warmup):
+        step()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for a, b in pairs:
+        a.record()
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / steps
+    ts = sorted(a.elapsed_time(b) * 1e3 for a, b in pairs)
+    _, _, npp = pkg.moe_align_block_size(inp.topk_ids, 64, shape.E_total)
+    P = M * inp.topk_ids.shape[1]
+    ids_cpu = inp.topk_ids.cpu()
+    ops, nbytes = pkg.inputs.algorithmic_ops(shape, M), pkg.inputs.algorithmic_bytes(shape, M, ids_cpu)
+    line = {"shape": shape_name, "M": M, "routing": shape.routing + (" + shared expert" if shape.shared_expert else ""),
+            "us": t * 1e6, "call_us_p50": ts[len(ts) // 2], "tokens_per_s": M / t,
+            "n_active_experts": int(torch.unique(ids_cpu).numel()), "padded_rows_over_pairs": int(npp.cpu()) / P,
+            "layer_hbm_frac": nbytes / t / PEAK_HBM_BPS, "layer_mfma_frac": ops / t / PEAK_INT8_OPS,
+            "bound": "hbm" if nbytes / PEAK_HBM_BPS >= ops / PEAK_INT8_OPS else "mfma"}
+    if cpu:
+        # only the experts this batch routes to travel to the host (ids remapped), so the checker does the same
+        # arithmetic on a few GB instead of the whole layer
+        used = torch.unique(ids_cpu.to(torch.int64))
+        remap = torch.full((shape.E_total,), -1, dtype=torch.int64)
+        remap[used] = torch.arange(used.numel())
+        dev_used = used.to("cuda:0")
+        args = (inp.hidden_states.cpu(), inp.w1[dev_used].cpu(), inp.w2[dev_used].cpu(), inp.topk_weights.cpu(),
+                remap[ids_cpu.to(torch.int64)].to(torch.int32), inp.w1_scale[dev_used].cpu(), inp.w2_scale[dev_used].cpu())
+        t0 = time.perf_counter()
+        oracle.native_w8a8_moe(*args)
+        tc = time.perf_counter() - t0
+        line["cpu"] = {"tokens_per_s": M / tc, "s": tc, "cores": torch.get_num_threads(), "kind": "port",
+                       "sample": "whole batch, one pass, no warm-up"}
+    del inp
+    torch.cuda.empty_cache()
+    return line
+
+
 def cpu_baseline(oracle, torch, base, sample_m: int) -> dict:
     m = min(sample_m, base.hidden_states.shape[0])
     args = (base.hidden_states[:m], base.w1, base.w2, base.topk_weights[:m], base.topk_ids[:m],
@@ -441,6 +538,7 @@ def main() -> int:
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-decode-mix", action="store_true")
+    ap.add_argument("--no-other-shapes", action="store_true")
     ap.add_argument("--decode-layers", type=int, default=48)
     ap.add_argument("--decode-steps", type=int, default=500)
     ap.add_argument("--cpu-sample", type=int, default=4096, help="tokens of the workload the CPU baseline runs")
@@ -472,8 +570,8 @@ def main() -> int:
         if hbm_bound:
             roof = {"bound": "hbm", "achieved": k_bytes / t_k / 1e9, "peak": PEAK_HBM_BPS / 1e9, "unit": "GB/s"}
         else:
-            roof = {"bound": "mfma", "achieved": k_ops / t_k / 1e12, "peak": PEAK_INT8_OPS / 1e12, "unit": "TFLOP/s",
-                    "note": "int8 TOP/s against the dense INT8 MFMA peak"}
+            roof = {"bound": "mfma", "achieved": k_ops / t_k / 1e12, "peak": PEAK_INT8_OPS / 1e12, "unit": "TOP/s",
+                    "note": "int8 operations per second against the dense INT8 MFMA peak"}
         roof["frac"] = roof["achieved"] / roof["peak"]
         roof["kernel"] = "gemm gate_up + SiLU*mul"
         roof["kernel_us"] = t_k * 1e6
@@ -540,8 +638,14 @@ def main() -> int:
         out["hbm_ceiling"] = time_hbm_ceiling(torch)
         if not args.no_decode_mix:
             out["decode_mix"] = time_decode_mix(pkg, torch, args.shape, args.decode_layers, args.decode_steps)
+    oracle = None if args.no_cpu else importlib.import_module("oracle.moe_i8_oracle")
+    if not args.no_sweep and not args.no_other_shapes:
+        out["other_shapes"] = [
+            time_other_shape(pkg, torch, oracle, name, M, max(args.steps // 2, 5), max(args.warmup // 2, 2),
+                             cpu=oracle is not None and i < 2)
+            for name, sizes in OTHER_SHAPES for i, M in enumerate(sizes)
+        ]
     if not args.no_cpu:
-        oracle = importlib.import_module("oracle.moe_i8_oracle")
         out["cpu_baseline"] = cpu_baseline(oracle, torch, base_headline, args.cpu_sample)
     print(json.dumps(out))
     return 0

@@ -250,17 +250,6 @@ int moe_i8_w8a8_mlp(const void* x, const int8_t* w13, const float* w13_scale, co
                     const float* w2_scale, void* out, int64_t m, int hidden, int inter, void* workspace,
                     int64_t workspace_bytes, int variant, void* stream);
 
-/*
- * Measurement aid with no counterpart in the reference: launches a register-only
- * v_mfma_i32_32x32x32_i8 loop (`iters` rounds of 8 instructions per wavefront, 8 wavefronts per
- * workgroup) on `workgroups` workgroups, with constant (random_operands = 0) or pseudo-random operand
- * bits.  The caller times the launch; moe_i8_probe_mfma_ops gives the int8 operations it performs.
- * The two rates bracket what the board's power limit leaves of the published int8 peak for a GEMM on
- * real data.  sink: device buffer of workgroups * 2048 bytes (written, never read).
- */
-double moe_i8_probe_mfma_ops(int workgroups, int iters);
-int moe_i8_probe_mfma(int random_operands, int workgroups, int iters, void* sink, int64_t sink_bytes, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

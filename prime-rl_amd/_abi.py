@@ -7,11 +7,12 @@ built, or exports fewer symbols than the header declares, importing callers get 
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
 from pathlib import Path
 
 PKG_DIR = Path(__file__).resolve().parent
 LIB_PATH = PKG_DIR / "libmoe_i8.so"
+PROBE_LIB_PATH = PKG_DIR / "libmoe_i8_probe.so"  # benchmark aid, not part of the product ABI
 
 OK = 0
 EINVAL, EWORKSPACE, ELAUNCH, EUNSUPPORTED = -1, -2, -3, -4
@@ -33,8 +34,6 @@ SIGNATURES = {
         c_int,
         [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int64, _P, _P],
     ),
-    "moe_i8_probe_mfma_ops": (c_double, [c_int, c_int]),
-    "moe_i8_probe_mfma": (c_int, [c_int, c_int, c_int, _P, c_int64, _P]),
     "moe_i8_scaled_int8_quant": (c_int, [_P, c_int, c_int64, c_int64, c_int64, _P, _P, _P]),
     "moe_i8_dense_workspace_bytes": (c_int64, [c_int64, c_int, c_int]),
     "moe_i8_w8a8_linear": (c_int, [_P, _P, _P, _P, c_int64, c_int, c_int, _P, c_int64, c_int, _P]),

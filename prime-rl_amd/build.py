@@ -11,7 +11,8 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libmoe_i8.so"
-SOURCES = ["align.hip", "quant.hip", "sum.hip", "router.hip", "gemm_stream.hip", "gemm_tile.hip", "gemm_narrow.hip", "probe.hip", "api.hip"]
+SOURCES = ["align.hip", "quant.hip", "sum.hip", "router.hip", "gemm_stream.hip", "gemm_tile.hip", "gemm_narrow.hip", "api.hip"]
+PROBE_LIB_PATH = PKG_DIR / "libmoe_i8_probe.so"  # the benchmark's MFMA rate probe, a library of its own
 
 # packed-fp32 VALU ops are switched off for all device code (hipcc's host pass warns that it does
 # not know the feature; that is harmless).
@@ -46,6 +47,7 @@ def build_library(verbose: bool = False) -> Path:
     objdir = PKG_DIR / "build"
     objdir.mkdir(exist_ok=True)
     objs = [objdir / (Path(s).stem + ".o") for s in SOURCES]
+    probe_obj = objdir / "probe.o"
 
     def compile_one(pair):
         src, obj = pair
@@ -54,11 +56,14 @@ def build_library(verbose: bool = False) -> Path:
             print(" ".join(cmd), flush=True)
         _run(cmd)
 
-    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
-        list(pool.map(compile_one, zip(SOURCES, objs)))
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES) + 1)) as pool:
+        list(pool.map(compile_one, zip([*SOURCES, "probe.hip"], [*objs, probe_obj])))
     tmp = LIB_PATH.with_suffix(".so.tmp")
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(tmp)])
     os.replace(tmp, LIB_PATH)
+    tmp = PROBE_LIB_PATH.with_suffix(".so.tmp")
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", str(probe_obj), "-o", str(tmp)])
+    os.replace(tmp, PROBE_LIB_PATH)
     return LIB_PATH
 
 

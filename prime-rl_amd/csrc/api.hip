@@ -744,18 +744,4 @@ int moe_i8_w8a8_mlp(const void* x, const int8_t* w13, const float* w13_scale, co
                           c.cap, out, variant, stream);
 }
 
-double moe_i8_probe_mfma_ops(int workgroups, int iters) {
-  return workgroups > 0 && iters > 0 ? moe_i8::mfma_probe_ops(workgroups, iters) : 0.0;
-}
-
-int moe_i8_probe_mfma(int random_operands, int workgroups, int iters, void* sink, int64_t sink_bytes, void* stream) {
-  if (workgroups < 1 || workgroups > 65535 || iters < 1) return fail(MOE_I8_EINVAL, "workgroups in [1, 65535], iters >= 1");
-  if (!sink || sink_bytes < moe_i8::mfma_probe_sink_bytes(workgroups))
-    return fail(MOE_I8_EWORKSPACE, "sink holds %lld bytes, %lld needed", (long long)sink_bytes,
-                (long long)moe_i8::mfma_probe_sink_bytes(workgroups));
-  return check_launch(moe_i8::launch_mfma_probe(random_operands != 0, workgroups, iters, static_cast<int32_t*>(sink),
-                                                static_cast<hipStream_t>(stream)),
-                      "mfma_probe");
-}
-
 }  // extern "C"

@@ -1,4 +1,5 @@
-// Measurement aid: a register-only v_mfma_i32_32x32x32_i8 loop on every compute unit.
+// Measurement aid, built into its own library (libmoe_i8_probe.so) that only the benchmark loads:
+// a register-only v_mfma_i32_32x32x32_i8 loop on every compute unit.
 //
 // The published int8 peak assumes the full shader clock.  Under the board's power limit the clock the
 // matrix pipes sustain depends on how much the operand bits toggle, so the rate reached with
@@ -68,3 +69,18 @@ hipError_t launch_mfma_probe(bool random_operands, int workgroups, int iters, in
 }
 
 }  // namespace moe_i8
+
+// C entry points of the probe library.  sink: device buffer of moe_i8_probe_sink_bytes(workgroups)
+// bytes (written, never read); returns 0 or a HIP error code.
+extern "C" {
+long long moe_i8_probe_sink_bytes(int workgroups) { return moe_i8::mfma_probe_sink_bytes(workgroups); }
+double moe_i8_probe_mfma_ops(int workgroups, int iters) {
+  return workgroups > 0 && iters > 0 ? moe_i8::mfma_probe_ops(workgroups, iters) : 0.0;
+}
+int moe_i8_probe_mfma(int random_operands, int workgroups, int iters, void* sink, long long sink_bytes, void* stream) {
+  if (workgroups < 1 || workgroups > 65535 || iters < 1 || !sink || sink_bytes < moe_i8::mfma_probe_sink_bytes(workgroups))
+    return (int)hipErrorInvalidValue;
+  return (int)moe_i8::launch_mfma_probe(random_operands != 0, workgroups, iters, static_cast<int32_t*>(sink),
+                                        static_cast<hipStream_t>(stream));
+}
+}

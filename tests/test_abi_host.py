@@ -100,10 +100,6 @@ def test_c_abi_rejects_bad_arguments_without_launching(pra):
     assert lib.moe_i8_sum(None, None, 0, 2, 64, None) == abi.OK
     assert lib.moe_i8_fused_experts(p, p, p, p, p, p, p, p, 4, 2, 4, 128, 64, 64, None, 0, 0, None) == abi.EINVAL
     assert lib.moe_i8_fused_experts(p, p, p, p, p, p, p, p, 4, 2, 4, 100, 64, 64, p, 1 << 30, 0, None) == abi.EINVAL
-    # the MFMA rate probe of the benchmark
-    assert lib.moe_i8_probe_mfma(1, 0, 10, p, 1 << 20, None) == abi.EINVAL
-    assert lib.moe_i8_probe_mfma(1, 256, 10, p, 256 * 2048 - 1, None) == abi.EWORKSPACE
-    assert lib.moe_i8_probe_mfma_ops(256, 10) == 256 * 8 * 10 * 8 * 65536.0
 
 
 def test_python_wrappers_refuse_cpu_tensors_and_unsupported_modes(pra):
