@@ -40,8 +40,10 @@ extern "C" {
 /* GEMM kernel families; MOE_I8_GEMM_AUTO picks by rows-per-expert. */
 #define MOE_I8_GEMM_AUTO 0
 #define MOE_I8_GEMM_STREAM 1 /* weights streamed global->registers, 16-row MFMA sub-tiles (decode) */
-#define MOE_I8_GEMM_TILE 2   /* LDS-staged double-buffered tiles, 32x32x32 MFMA (prefill) */
+#define MOE_I8_GEMM_TILE 2   /* LDS-staged tiles, 32x32x32 MFMA (prefill); geometry by rows per expert */
 #define MOE_I8_GEMM_NARROW 3 /* 64-row tiles, three LDS stages kept in flight (tens of rows per expert) */
+#define MOE_I8_GEMM_TILE_WIDE 4 /* the LDS-tiled family with 256-row tiles and two stages (many rows per expert) */
+#define MOE_I8_GEMM_TILE_DEEP 5 /* the LDS-tiled family with 128-row tiles and three stages (around 100 rows per expert) */
 
 /* Router score functions (reference TokenChoiceTopKRouter.score_func). */
 #define MOE_I8_SCORE_SOFTMAX 0      /* softmax over all experts */

@@ -46,7 +46,10 @@ __all__ = [
 ]
 
 DEFAULT_BLOCK_SIZE_M = 64
-_VARIANTS = {"auto": _abi.GEMM_AUTO, "stream": _abi.GEMM_STREAM, "tile": _abi.GEMM_TILE, "narrow": _abi.GEMM_NARROW}
+_VARIANTS = {
+    "auto": _abi.GEMM_AUTO, "stream": _abi.GEMM_STREAM, "tile": _abi.GEMM_TILE, "narrow": _abi.GEMM_NARROW,
+    "tile_wide": _abi.GEMM_TILE_WIDE, "tile_deep": _abi.GEMM_TILE_DEEP,
+}
 # Default workspaces, one per (device, stream) that has called without a caller-owned one: a small
 # LRU (a process has a handful of forward streams) guarded by a lock.  Entries are only ever created or
 # grown outside HIP graph capture, so a captured graph never holds a pointer that a later call frees:

@@ -45,19 +45,36 @@ int check_gemm_common(const void* a_q, const void* w, const int32_t* sorted, con
   if (k < 64 || k % 64) return fail(MOE_I8_EINVAL, "reduction length (%d) must be a positive multiple of 64", k);
   if (sorted_cap < moe_i8_sorted_capacity(num_pairs, num_experts, block_size))
     return fail(MOE_I8_EWORKSPACE, "sorted_token_ids capacity %lld too small", (long long)sorted_cap);
-  if (variant != MOE_I8_GEMM_AUTO && variant != MOE_I8_GEMM_STREAM && variant != MOE_I8_GEMM_TILE &&
-      variant != MOE_I8_GEMM_NARROW)
+  if (variant < MOE_I8_GEMM_AUTO || variant > MOE_I8_GEMM_TILE_DEEP)
     return fail(MOE_I8_EINVAL, "unknown GEMM variant %d", variant);
   return MOE_I8_OK;
 }
 
 constexpr int kStreamRowsPerExpert = 8;
-constexpr int kNarrowRowsPerExpert = 56;
 
-// Which family a launch goes to (one of the MOE_I8_GEMM_* constants, never AUTO); -1 with the error
-// set if a family was demanded for a shape it does not handle.
-int picks_family(const moe_i8::GemmArgs& g, int variant) {
-  if (variant == MOE_I8_GEMM_TILE) {
+int tile_geometry_of(int variant) {
+  return variant == MOE_I8_GEMM_TILE_WIDE ? moe_i8::kTileWide
+         : variant == MOE_I8_GEMM_TILE_DEEP ? moe_i8::kTileDeep
+                                            : moe_i8::kTileAuto;
+}
+
+// Routed rows per expert up to which the narrow tiles beat the deep geometry of the LDS-tiled family.
+// The narrow tiles (two small workgroups per compute unit, 64 x 128 tasks) start up faster and
+// balance better; the deep tiles stream an expert's weights once for up to 128 rows and sustain
+// more bytes in flight, which counts the more the longer a launch runs.  Measured crossovers, with
+// the weight bytes of the launch: 0.2-0.4 GB (Qwen3-30B-A3B) 44-48 rows, 0.7-1.5 GB (GLM-4.5-Air)
+// 22-30, 3.8-7.5 GB (DeepSeek-V3) at most 8.
+int narrow_rows_per_expert(const moe_i8::GemmArgs& g) {
+  const int64_t weight_bytes = (int64_t)g.num_experts * g.n * g.k;
+  return weight_bytes < (512ll << 20) ? 48 : weight_bytes < (2048ll << 20) ? 24 : 12;
+}
+
+// Which family a launch goes to (MOE_I8_GEMM_STREAM, _TILE or _NARROW); -1 with the error set if a
+// family was demanded for a shape it does not handle.
+int picks_family(const moe_i8::GemmArgs& g0, int variant) {
+  moe_i8::GemmArgs g = g0;
+  g.tile_geometry = tile_geometry_of(variant);
+  if (variant == MOE_I8_GEMM_TILE || variant == MOE_I8_GEMM_TILE_WIDE || variant == MOE_I8_GEMM_TILE_DEEP) {
     if (!moe_i8::gemm_tile_supports(g))
       return fail(MOE_I8_EUNSUPPORTED, "tile GEMM does not support this shape"), -1;
     return MOE_I8_GEMM_TILE;
@@ -68,23 +85,25 @@ int picks_family(const moe_i8::GemmArgs& g, int variant) {
     return MOE_I8_GEMM_NARROW;
   }
   if (variant == MOE_I8_GEMM_STREAM) return MOE_I8_GEMM_STREAM;
-  // Measured crossovers on the Qwen3-30B-A3B shape, in routed rows per expert: with evenly spread
-  // routing the streaming family wins while a block mostly holds one 16-row sub-tile (up to about
-  // 12), the narrow tiles while most experts hold a single 64-row block (up to about 56), the wide
-  // LDS tiles beyond.  The streaming family reads an expert's weights once per 16 (or 32) of its
-  // rows, so skewed routing costs it far more than the tiled families (a few experts with a
-  // hundred rows double its time); the first crossover is therefore set lower, at 8, where the
-  // narrow tiles lose 2 % or less on even routing.
+  // Measured crossovers, in routed rows per expert.  With evenly spread routing the streaming
+  // family wins while a block mostly holds one 16-row sub-tile (up to about 12); it reads an
+  // expert's weights once per 16 (or 32) of its rows, so skewed routing costs it far more than the
+  // tiled families (a few experts with a hundred rows double its time), and the first crossover is
+  // therefore set lower, at 8, where the narrow tiles lose 2 % or less on even routing.  Then the
+  // narrow tiles while most experts hold a single 64-row block, then the LDS-tiled family (which
+  // picks its own geometry).
   const int64_t rows_x_experts = g.num_pairs;
   if (rows_x_experts <= (int64_t)kStreamRowsPerExpert * g.num_experts) return MOE_I8_GEMM_STREAM;
-  if (rows_x_experts <= (int64_t)kNarrowRowsPerExpert * g.num_experts && moe_i8::gemm_narrow_supports(g))
+  if (rows_x_experts <= (int64_t)narrow_rows_per_expert(g) * g.num_experts && moe_i8::gemm_narrow_supports(g))
     return MOE_I8_GEMM_NARROW;
   if (moe_i8::gemm_tile_supports(g)) return MOE_I8_GEMM_TILE;
   return moe_i8::gemm_narrow_supports(g) ? MOE_I8_GEMM_NARROW : MOE_I8_GEMM_STREAM;
 }
 
-int run_gemm(const moe_i8::GemmArgs& g, int variant, hipStream_t stream) {
-  if (g.num_pairs == 0) return MOE_I8_OK;
+int run_gemm(const moe_i8::GemmArgs& g0, int variant, hipStream_t stream) {
+  if (g0.num_pairs == 0) return MOE_I8_OK;
+  moe_i8::GemmArgs g = g0;
+  g.tile_geometry = tile_geometry_of(variant);
   switch (picks_family(g, variant)) {
     case MOE_I8_GEMM_TILE: return check_launch(moe_i8::launch_gemm_tile(g, stream), "gemm_tile");
     case MOE_I8_GEMM_NARROW: return check_launch(moe_i8::launch_gemm_narrow(g, stream), "gemm_narrow");

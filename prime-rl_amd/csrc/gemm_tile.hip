@@ -1,26 +1,35 @@
-// Grouped int8 GEMM for gfx950, LDS-tiled family (many rows per expert: prefill).
+// Grouped int8 GEMM for gfx950, LDS-tiled family (prefill: from a few dozen routed rows per expert up).
 //
 // Persistent workgroups (one per CU, 512 threads = 8 wavefronts) walk a list of tiles.  A tile is
-// up to 256 token rows of ONE expert (up to four 64-row moe_align blocks, aligned to the start of
-// the expert's segment) x 256 weight rows (output channels); the reduction runs in steps of 128
-// bytes.  Wavefront w owns token sub-block w / 2 (64 rows) x channel half w % 2 (128 channels) as
-// 2 x 4 v_mfma_i32_32x32x32_i8 tiles (128 accumulator VGPRs).  The MFMA is used "transposed"
-// (A operand = weight rows, B operand = token rows), so a lane ends up with runs of 4 consecutive
-// channels of one token.
+// a run of 64-row moe_align sub-blocks of ONE expert (aligned to the start of the expert's segment)
+// x 256 weight rows (output channels); the reduction runs in steps of 128 bytes.  The MFMA
+// (v_mfma_i32_32x32x32_i8) is used "transposed" (A operand = weight rows, B operand = token rows),
+// so a lane ends up with runs of 4 consecutive channels of one token.
+//
+// Two geometries (template parameter DEEP):
+//  * wide: up to 256 token rows per tile, two 64 KB LDS stages, loads one step ahead.  Wavefront w
+//    owns token sub-block w / 2 x channel half w % 2 as 4 x 2 MFMA tiles (128 accumulator VGPRs).
+//    Bound by the matrix pipe; a weight tile is reused by up to four sub-blocks.
+//  * deep: up to 128 token rows per tile, a ring of three 48 KB stages, loads two steps ahead.  With
+//    few rows per expert a step holds little arithmetic and the kernel is bound by the weight stream
+//    from HBM, i.e. by the bytes a compute unit keeps in flight.  All eight wavefronts multiply in
+//    every task: with two active sub-blocks wavefront w owns sub-block w / 4 and a quarter of the
+//    channels, with one an eighth of the channels.
 //
 // Both operands go global -> LDS directly (global_load_lds_dwordx4: no staging registers, no
-// ds_write) into two 64 KB stages: while step s is multiplied the loads of step s+1 are in flight,
-// with one s_barrier per step and explicit vmcnt waits.  Every wavefront-level load covers 8 rows
-// x 128 contiguous bytes, i.e. whole cache lines.  LDS rows are 128 bytes; the 16-byte chunk index
-// is XOR-swizzled with row bits so that the MFMA-layout reads (32 consecutive rows, same chunk)
-// spread over all banks; because a load fills LDS linearly the swizzle is applied to the global
-// source address of each lane.
+// ds_write), with one s_barrier per step and explicit vmcnt waits.  Every wavefront-level load
+// covers 8 rows x 128 contiguous bytes, i.e. whole cache lines.  LDS rows are 128 bytes; the 16-byte
+// chunk index is XOR-swizzled with row bits so that the MFMA-layout reads (32 consecutive rows, same
+// chunk) spread over all banks; because a load fills LDS linearly the swizzle is applied to the
+// global source address of each lane.
 //
 // The tile list is derived inside the kernel from expert_ids (block -> expert, ascending): every
 // workgroup scans it once into LDS.  Tasks (tile, channel tile) are numbered channel tile fastest
 // and split into 8 contiguous ranges, one per XCD (workgroup id % 8), so that the workgroups
 // running on one XCD at a time share token rows and expert weights in that XCD's L2.  The first
 // loads of the next task are issued before the epilogue of the current one.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace moe_i8 {
@@ -28,12 +37,22 @@ namespace {
 
 constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / kWave;
-constexpr int kTileTok = 256;  // token rows per tile
 constexpr int kBN = 256;       // weight rows per tile
 constexpr int kBK = 128;       // reduction bytes per step
 constexpr int kTokOffset = kBN * kBK;
-constexpr int kStageBytes = (kBN + kTileTok) * kBK;  // 64 KB
-constexpr int kMaxTiles = 6144;                      // capacity of the in-LDS tile list
+
+// Two geometries.  Wide: tiles of up to 256 token rows, two 64 KB stages (loads one step ahead).
+// Deep: tiles of up to 128 token rows, a ring of three 48 KB stages (loads two steps ahead): with
+// few rows per expert a step holds little arithmetic, and what bounds the kernel is how many bytes
+// of the weight stream a compute unit keeps in flight.
+template <bool DEEP>
+struct Geometry {
+  static constexpr int kTileTok = DEEP ? 128 : 256;               // token rows per tile
+  static constexpr int kSlots = DEEP ? 3 : 2;                     // LDS stages
+  static constexpr int kStageBytes = (kBN + kTileTok) * kBK;      // 48 KB | 64 KB
+  static constexpr int kMaxTiles = DEEP ? 2048 : 6144;            // capacity of the in-LDS tile list
+  static constexpr int kTokLoads = kTileTok / 64;                 // wave-level loads of 8 token rows per wavefront and step
+};
 constexpr int kXcds = 8;
 constexpr int kGroupTiles = 8;  // token tiles of one expert whose tasks are interleaved per channel tile
 
@@ -117,7 +136,7 @@ __device__ __forceinline__ void block_scan(int v, int* wave_part, int& incl, int
 // Tiles start at multiples of `per_tile` blocks inside each run of equal expert ids and never cross
 // a run; up to kGroupTiles consecutive tiles of a run form a group.  scratch holds nblocks ints.
 __device__ int build_tile_list(const int32_t* __restrict__ expert_ids, int nblocks, int per_tile, int* scratch,
-                               int* wave_part, uint32_t* tile_desc, int* total_out) {
+                               int* wave_part, uint32_t* tile_desc, int* total_out, int max_tiles) {
   const int tid = threadIdx.x;
   for (int j = tid; j < nblocks; j += kThreads) scratch[j] = expert_ids[j];
   __syncthreads();
@@ -145,12 +164,12 @@ __device__ int build_tile_list(const int32_t* __restrict__ expert_ids, int nbloc
       int nb = 1;
       while (nb < per_tile && j + nb < nblocks && scratch[j + nb] == scratch[j]) ++nb;
       // bits 0-15 first block, 16-19 blocks, 20-22 rank of the tile inside its group, 24-27 group size
-      if (t < kMaxTiles)
+      if (t < max_tiles)
         tile_desc[t] = (uint32_t)j | ((uint32_t)nb << 16) | ((uint32_t)(((j - cur) / per_tile) % kGroupTiles) << 20);
       ++t;
     }
   }
-  if (tid == kThreads - 1) *total_out = incl_leaders < kMaxTiles ? incl_leaders : kMaxTiles;
+  if (tid == kThreads - 1) *total_out = incl_leaders < max_tiles ? incl_leaders : max_tiles;
   __syncthreads();
   // Groups: up to kGroupTiles consecutive tiles of one expert.  The leader of a group counts its
   // members and writes the size into all of them.
@@ -178,10 +197,12 @@ struct TaskLoads {
   uint32_t xoff[4];     // per lane: byte offset of its chunk of token row i from a_q
 };
 
-// Lane fills LDS slot (lane & 7) of row 32 * wave + 8 * i + (lane >> 3): it fetches the logical
-// chunk (lane & 7) ^ swizzle(row) of that row, and swizzle(row) = (lane >> 3) ^ (i & 1).
-template <int MODE>
+// Weights: lane fills LDS slot (lane & 7) of row 32 * wave + 8 * i + (lane >> 3): it fetches the logical
+// chunk (lane & 7) ^ swizzle(row) of that row, and swizzle(row) = (lane >> 3) ^ (i & 1).  Token rows
+// likewise, of row (8 * kTokLoads) * wave + 8 * i + (lane >> 3).
+template <int MODE, bool DEEP>
 __device__ __forceinline__ void setup_loads(const TileParams& p, const Task& tk, int wave, int lane, TaskLoads& ld) {
+  constexpr int kTokLoads = Geometry<DEEP>::kTokLoads;
   const int K = p.K;
   const int inter = p.N / 2;
 #pragma unroll
@@ -197,24 +218,32 @@ __device__ __forceinline__ void setup_loads(const TileParams& p, const Task& tk,
       n = ch < p.N ? ch : p.N - 1;
     }
     ld.woff[i] = (uint32_t)n * (uint32_t)K + chunk;
-    uint32_t arow = 0;
-    if ((wave >> 1) < tk.nsub) {
-      const int32_t tok = p.sorted_ids[tk.slot0 + row];
-      if (tok >= 0 && tok < p.P) arow = (uint32_t)(tok / p.row_div);
+    if (i < kTokLoads) {
+      const int trow = 8 * kTokLoads * wave + 8 * i + (lane >> 3);
+      uint32_t arow = 0;
+      if ((trow >> 6) < tk.nsub) {
+        const int32_t tok = p.sorted_ids[tk.slot0 + trow];
+        if (tok >= 0 && tok < p.P) arow = (uint32_t)(tok / p.row_div);
+      }
+      ld.xoff[i] = arow * (uint32_t)K + chunk;
     }
-    ld.xoff[i] = arow * (uint32_t)K + chunk;
   }
   ld.wbase = p.w + (int64_t)tk.e * p.N * K;
 }
 
+// `tokens`: this wavefront's token rows belong to an active sub-block.  The deep geometry issues the
+// token loads regardless (rows of inactive sub-blocks fetch row 0), so that every wavefront has the
+// same number of loads in flight per step and the counted waits of the ring hold for all of them.
+template <bool DEEP>
 __device__ __forceinline__ void issue_stage_loads(const TaskLoads& ld, const int8_t* a_q, uint32_t stage_addr,
                                                   int wave, int koff, bool tokens) {
+  constexpr int kTokLoads = Geometry<DEEP>::kTokLoads;
 #pragma unroll
   for (int i = 0; i < 4; ++i) load_to_lds_16(ld.wbase + koff, ld.woff[i], stage_addr + (wave * 4 + i) * 1024);
-  if (tokens) {
+  if (DEEP || tokens) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      load_to_lds_16(a_q + koff, ld.xoff[i], stage_addr + kTokOffset + (wave * 4 + i) * 1024);
+    for (int i = 0; i < kTokLoads; ++i)
+      load_to_lds_16(a_q + koff, ld.xoff[i], stage_addr + kTokOffset + (wave * kTokLoads + i) * 1024);
   }
 }
 
@@ -224,8 +253,41 @@ struct TileReads {
   int chunk[4];  // swizzled byte offset of logical chunk 2 * kk + (lane >> 5)
 };
 
-__device__ __forceinline__ void multiply_stage(const TileReads& rd, const char* stage, v16i (&acc)[4][2]) {
-  v4i a[4][4], b[4][2];
+// How the eight wavefronts share a task.  A task with NCI = 4 has three or four active 64-row
+// sub-blocks: wavefront w owns sub-block w / 2 and half of the channels (4 MFMA tiles of 32 weight
+// rows, twice 32 token rows).  With two active sub-blocks (NCI = 2) it owns sub-block w / 4 and a
+// quarter of the channels, with one (NCI = 1) an eighth of the channels: every wavefront multiplies
+// in every task, so a tile with few rows costs its loads and not the serial MFMA chain of the one
+// or two wavefronts its rows would otherwise belong to.
+template <int MODE, int NCI>
+__device__ __forceinline__ void make_reads(int wave, int lane, TileReads& rd) {
+  constexpr int kParts = 8 / NCI;
+  const int tg = wave / kParts;
+  const int cpart = wave % kParts;
+  const int lrow = lane & 31;
+#pragma unroll
+  for (int ci = 0; ci < NCI; ++ci) {
+    int row;
+    if constexpr (MODE == kGateUpSilu) {
+      // LDS rows 0..127 hold gate channels, 128..255 the matching up channels
+      if constexpr (NCI == 4)
+        row = (ci < 2 ? 0 : 128) + cpart * 64 + (ci & 1) * 32 + lrow;
+      else if constexpr (NCI == 2)
+        row = ci * 128 + cpart * 32 + lrow;
+      else
+        row = (lrow < 16 ? 0 : 128 - 16) + cpart * 16 + lrow;  // 16 gate rows, then their 16 up rows
+    } else {
+      row = cpart * (NCI * 32) + ci * 32 + lrow;
+    }
+    rd.w_ld[ci] = row * kBK;
+  }
+#pragma unroll
+  for (int tj = 0; tj < 2; ++tj) rd.x_ld[tj] = kTokOffset + (tg * 64 + tj * 32 + lrow) * kBK;
+}
+
+template <int NCI>
+__device__ __forceinline__ void multiply_stage(const TileReads& rd, const char* stage, v16i (&acc)[NCI][2]) {
+  v4i a[4][NCI], b[4][2];
   // reads in the order the MFMAs consume them: b0 a0 | b1 | a1 | a2 | a3 per 32-byte sub-step
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk) {
@@ -233,50 +295,66 @@ __device__ __forceinline__ void multiply_stage(const TileReads& rd, const char* 
     a[kk][0] = *reinterpret_cast<const v4i*>(stage + rd.w_ld[0] + rd.chunk[kk]);
     b[kk][1] = *reinterpret_cast<const v4i*>(stage + rd.x_ld[1] + rd.chunk[kk]);
 #pragma unroll
-    for (int ci = 1; ci < 4; ++ci) a[kk][ci] = *reinterpret_cast<const v4i*>(stage + rd.w_ld[ci] + rd.chunk[kk]);
+    for (int ci = 1; ci < NCI; ++ci) a[kk][ci] = *reinterpret_cast<const v4i*>(stage + rd.w_ld[ci] + rd.chunk[kk]);
   }
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
-    for (int ci = 0; ci < 4; ++ci)
+    for (int ci = 0; ci < NCI; ++ci)
 #pragma unroll
       for (int tj = 0; tj < 2; ++tj)
         acc[ci][tj] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[kk][ci], b[kk][tj], acc[ci][tj], 0, 0, 0);
-  // Fine interleave, one group ahead: the first MFMA issues as soon as three operands are in and
-  // every later read is issued at least one MFMA group before its first use, so it is hidden
-  // behind MFMAs already queued (8 wavefronts share the LDS: a long burst of reads in front of the
-  // first MFMA would leave the matrix pipe idle at the start of every step).
-  __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);  // b0 a0 b1 of sub-step 0
+  if constexpr (NCI == 4) {
+    // Fine interleave, one group ahead: the first MFMA issues as soon as three operands are in and
+    // every later read is issued at least one MFMA group before its first use, so it is hidden
+    // behind MFMAs already queued (8 wavefronts share the LDS: a long burst of reads in front of the
+    // first MFMA would leave the matrix pipe idle at the start of every step).
+    __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);  // b0 a0 b1 of sub-step 0
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // a0 b0
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // a1
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // a0 b1
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // a2
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // a1
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // a3
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // a2
-    if (kk < 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // next b0 a0
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // a3
-    if (kk < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // next b1
+    for (int kk = 0; kk < 4; ++kk) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // a0 b0
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // a1
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // a0 b1
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // a2
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // a1
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // a3
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // a2
+      if (kk < 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // next b0 a0
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // a3
+      if (kk < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // next b1
+    }
   }
 }
 
-// acc[ci][tj][4q + r] is channel base(ci) + 8q + 4 * (lane >> 5) + r of token row
-// tb * 64 + tj * 32 + (lane & 31) of the tile.  The bf16 results are transposed through an 8 KB
-// LDS region private to the wavefront so that the global stores are 16 bytes per lane and cover
-// whole cache lines of an output row (rows of 16-byte chunks, chunk index XOR-swizzled with the row
-// so that neither the 8-byte writes nor the 16-byte reads pile up on a bank).
-template <int MODE>
-__device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, int chh, int tb, int lane,
-                                         v16i (&acc)[4][2], char* wave_lds, float* wave_scales) {
+// acc[ci][tj][4q + r] is weight row 32 * ci + 8q + 4 * (lane >> 5) + r of the wavefront's MFMA tiles
+// and token row tg * 64 + tj * 32 + (lane & 31) of the tile.  The bf16 results are transposed through
+// an LDS region private to the wavefront (at most 8 KB) so that the global stores are 16 bytes per
+// lane and cover whole runs of an output row (rows of 16-byte chunks, chunk index XOR-swizzled with
+// the row so that neither the 8-byte writes nor the 16-byte reads pile up on a bank).
+template <int CPR>
+__device__ __forceinline__ int staging_swizzle(int row) {
+  // rows of CPR chunks: 16 / CPR rows span all banks, rows that far apart must differ in the swizzle
+  if constexpr (CPR >= 8)
+    return row & (CPR - 1);
+  else if constexpr (CPR == 4)
+    return (row >> 2) & 3;
+  else
+    return (row >> 3) & 1;
+}
+
+template <int MODE, int NCI>
+__device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, int wave, int lane, v16i (&acc)[NCI][2],
+                                         char* wave_lds, float* wave_scales) {
+  constexpr int kParts = 8 / NCI;
+  const int tg = wave / kParts;
+  const int cpart = wave % kParts;
   const int lrow = lane & 31;
   const int lhalf = lane >> 5;
   const int inter = p.N / 2;
   int32_t tok[2];
 #pragma unroll
   for (int tj = 0; tj < 2; ++tj) {
-    tok[tj] = p.sorted_ids[tk.slot0 + tb * 64 + tj * 32 + lrow];
+    tok[tj] = p.sorted_ids[tk.slot0 + tg * 64 + tj * 32 + lrow];
     if (tok[tj] < 0 || tok[tj] >= p.P) tok[tj] = -1;
   }
   if constexpr (MODE == kAccI32) {
@@ -285,22 +363,25 @@ __device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, in
       if (tok[tj] < 0) continue;
       int32_t* out = static_cast<int32_t*>(p.out) + (int64_t)tok[tj] * p.N;
 #pragma unroll
-      for (int ci = 0; ci < 4; ++ci)
+      for (int ci = 0; ci < NCI; ++ci)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int n = tk.nt * kBN + chh * 128 + ci * 32 + 8 * q + 4 * lhalf;
+          const int n = tk.nt * kBN + cpart * (NCI * 32) + ci * 32 + 8 * q + 4 * lhalf;
           if (n < p.N)
             *reinterpret_cast<v4i*>(out + n) =
                 v4i{acc[ci][tj][4 * q], acc[ci][tj][4 * q + 1], acc[ci][tj][4 * q + 2], acc[ci][tj][4 * q + 3]};
         }
     }
   } else if constexpr (MODE == kDown) {
+    constexpr int kChannels = NCI * 32;  // of this wavefront
+    constexpr int CPR = NCI * 4;         // 16-byte chunks per staged row
+    constexpr int kRowBytes = CPR * 16;
     const float* wsc = p.w_scale + (int64_t)tk.e * p.N;
-    const int n0 = tk.nt * kBN + chh * 128;  // first channel of this wavefront
-    // The 128 channel scales of this wavefront go through LDS: read from there they do not count
+    const int n0 = tk.nt * kBN + cpart * kChannels;  // first channel of this wavefront
+    // The channel scales of this wavefront go through LDS: read from there they do not count
     // as vector-memory loads, so the second half's arithmetic does not have to wait for the first
     // half's stores (the vector-memory counter retires in order).
-    {
+    if (2 * lane < kChannels) {
       const int n = n0 + 2 * lane;
       *reinterpret_cast<float2*>(wave_scales + 2 * lane) =
           n < p.N ? *reinterpret_cast<const float2*>(wsc + n) : make_float2(0.0f, 0.0f);
@@ -313,15 +394,15 @@ __device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, in
     }
 #pragma unroll
     for (int tj = 0; tj < 2; ++tj) {
-      // 32 token rows x 128 channels: rows of 256 bytes = 16 chunks
+      // 32 token rows x kChannels channels
 #pragma unroll
-      for (int ci = 0; ci < 4; ++ci) {
+      for (int ci = 0; ci < NCI; ++ci) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const float4 ws = *reinterpret_cast<const float4*>(wave_scales + ci * 32 + 8 * q + 4 * lhalf);
           const int v[4] = {acc[ci][tj][4 * q], acc[ci][tj][4 * q + 1], acc[ci][tj][4 * q + 2], acc[ci][tj][4 * q + 3]};
-          *reinterpret_cast<uint2*>(wave_lds + lrow * 256 + (((ci * 4 + q) ^ (lrow & 15)) * 16) + lhalf * 8) =
-              down_epilogue4(v, as[tj], ws, rw[tj]);
+          *reinterpret_cast<uint2*>(wave_lds + lrow * kRowBytes + (((ci * 4 + q) ^ staging_swizzle<CPR>(lrow)) * 16) +
+                                    lhalf * 8) = down_epilogue4(v, as[tj], ws, rw[tj]);
         }
       }
       // Before the first stores everything this wavefront has in flight is complete (its share of
@@ -329,10 +410,11 @@ __device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, in
       // stores are the only vector-memory work still pending when the next tile starts.
       if (tj == 0) wait_vmcnt<0>();
 #pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        const int row = r * 4 + (lane >> 4);
-        const int chunk = lane & 15;
-        const uint4 v = *reinterpret_cast<const uint4*>(wave_lds + row * 256 + ((chunk ^ (row & 15)) * 16));
+      for (int r = 0; r < CPR / 2; ++r) {
+        const int row = r * (64 / CPR) + lane / CPR;
+        const int chunk = lane % CPR;
+        const uint4 v =
+            *reinterpret_cast<const uint4*>(wave_lds + row * kRowBytes + ((chunk ^ staging_swizzle<CPR>(row)) * 16));
         const int32_t t = __shfl(tok[tj], row);
         const int n = n0 + chunk * 8;
         if (t >= 0 && n < p.N)
@@ -340,35 +422,42 @@ __device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, in
       }
     }
   } else {
+    constexpr int kChannels = NCI * 16;  // activation channels of this wavefront
+    constexpr int CPR = NCI * 2;
+    constexpr int kRowBytes = CPR * 16;
     const float* wsc = p.w_scale + (int64_t)tk.e * p.N;
-    const int n0 = tk.nt * 128 + chh * 64;  // first gate channel of this wavefront
-    // 64 token rows x 64 channels: rows of 128 bytes = 8 chunks
+    const int n0 = tk.nt * 128 + cpart * kChannels;  // first gate channel of this wavefront
+    // 64 token rows x kChannels channels
 #pragma unroll
     for (int tj = 0; tj < 2; ++tj) {
       const float as = tok[tj] >= 0 ? p.a_scale[tok[tj] / p.row_div] : 0.0f;
       const int row = tj * 32 + lrow;
 #pragma unroll
-      for (int ci = 0; ci < 2; ++ci)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = n0 + ci * 32 + 8 * q + 4 * lhalf;
-          const int ns = n < inter ? n : 0;
-          const float4 wg = *reinterpret_cast<const float4*>(wsc + ns);
-          const float4 wu = *reinterpret_cast<const float4*>(wsc + inter + ns);
-          const int g[4] = {acc[ci][tj][4 * q], acc[ci][tj][4 * q + 1], acc[ci][tj][4 * q + 2], acc[ci][tj][4 * q + 3]};
-          const int u[4] = {acc[ci + 2][tj][4 * q], acc[ci + 2][tj][4 * q + 1], acc[ci + 2][tj][4 * q + 2],
-                            acc[ci + 2][tj][4 * q + 3]};
-          *reinterpret_cast<uint2*>(wave_lds + row * 128 + (((ci * 4 + q) ^ (row & 7)) * 16) + lhalf * 8) =
-              silu_mul_epilogue4(g, u, as, wg, wu);
-        }
+      for (int c = 0; c < CPR; ++c) {
+        // gate rows sit in MFMA tile gi at 8 * gq, the matching up rows in tile ui at 8 * uq
+        constexpr int kHalfTiles = NCI >= 2 ? NCI / 2 : 1;
+        const int gi = NCI >= 2 ? c / 4 : 0;
+        const int gq = NCI >= 2 ? c % 4 : c;
+        const int ui = NCI >= 2 ? gi + kHalfTiles : 0;
+        const int uq = NCI >= 2 ? gq : c + 2;
+        const int n = n0 + c * 8 + 4 * lhalf;
+        const int ns = n < inter ? n : 0;
+        const float4 wg = *reinterpret_cast<const float4*>(wsc + ns);
+        const float4 wu = *reinterpret_cast<const float4*>(wsc + inter + ns);
+        const int g[4] = {acc[gi][tj][4 * gq], acc[gi][tj][4 * gq + 1], acc[gi][tj][4 * gq + 2], acc[gi][tj][4 * gq + 3]};
+        const int u[4] = {acc[ui][tj][4 * uq], acc[ui][tj][4 * uq + 1], acc[ui][tj][4 * uq + 2], acc[ui][tj][4 * uq + 3]};
+        *reinterpret_cast<uint2*>(wave_lds + row * kRowBytes + ((c ^ staging_swizzle<CPR>(row)) * 16) + lhalf * 8) =
+            silu_mul_epilogue4(g, u, as, wg, wu);
+      }
     }
     wait_vmcnt<0>();  // as in the down epilogue: only the stores below stay pending
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const int row = r * 8 + (lane >> 3);
-      const int chunk = lane & 7;
-      const uint4 v = *reinterpret_cast<const uint4*>(wave_lds + row * 128 + ((chunk ^ (row & 7)) * 16));
-      const int32_t t = __shfl(tok[r >> 2], row & 31);
+    for (int r = 0; r < CPR; ++r) {
+      const int row = r * (64 / CPR) + lane / CPR;
+      const int chunk = lane % CPR;
+      const uint4 v =
+          *reinterpret_cast<const uint4*>(wave_lds + row * kRowBytes + ((chunk ^ staging_swizzle<CPR>(row)) * 16));
+      const int32_t t = __shfl(tok[(r * (64 / CPR)) >> 5], row & 31);
       const int n = n0 + chunk * 8;
       if (t >= 0 && n < inter)
         __builtin_nontemporal_store(v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w}, reinterpret_cast<v4i*>(static_cast<uint16_t*>(p.out) + (int64_t)t * inter + n));
@@ -376,10 +465,12 @@ __device__ __forceinline__ void epilogue(const TileParams& p, const Task& tk, in
   }
 }
 
-template <int MODE>
+template <int MODE, bool DEEP>
 __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(TileParams p) {
-  __shared__ __align__(16) char stages[2 * kStageBytes];
-  __shared__ uint32_t tile_desc[kMaxTiles];
+  using G = Geometry<DEEP>;
+  constexpr int kStageBytes = G::kStageBytes;
+  __shared__ __align__(16) char stages[G::kSlots * kStageBytes];
+  __shared__ uint32_t tile_desc[G::kMaxTiles];
   __shared__ int wave_part[kWaves];
   __shared__ __align__(16) float channel_scales[kWaves * 128];
   __shared__ int total_tiles;
@@ -387,36 +478,23 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(TileParams p) {
   const int t = threadIdx.x;
   const int lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-  const int tb = wave >> 1;  // token sub-block of this wavefront
-  const int chh = wave & 1;  // channel half
+  const int load_sub = wave * G::kTokLoads / 8;  // token sub-block whose rows this wavefront loads
   const int nk = p.K / kBK;
 
   const int npp = *p.npp;
   const int nblocks = npp / p.B;
   const int sub_per_block = p.B / 64;
-  const int ntile = build_tile_list(p.expert_ids, nblocks, kTileTok / p.B, reinterpret_cast<int*>(stages), wave_part,
-                                    tile_desc, &total_tiles);
+  const int ntile = build_tile_list(p.expert_ids, nblocks, G::kTileTok / p.B, reinterpret_cast<int*>(stages),
+                                    wave_part, tile_desc, &total_tiles, G::kMaxTiles);
   const int total = ntile * p.ntiles;
   const int per_xcd = (total + kXcds - 1) / kXcds;
   const int xcd = blockIdx.x % kXcds;
   const int stride = gridDim.x / kXcds;
 
   // ---- MFMA operand reads: lane feeds row (lane & 31), 16-byte chunk 2 * kk + (lane >> 5) ----
-  const int lrow = lane & 31;
-  const int lsw = swizzle_of_row(lrow);
+  const int lsw = swizzle_of_row(lane & 31);
   const int lhalf = lane >> 5;
   TileReads rd;
-#pragma unroll
-  for (int ci = 0; ci < 4; ++ci) {
-    int row0;
-    if constexpr (MODE == kGateUpSilu)
-      row0 = (ci < 2 ? 0 : 128) + chh * 64 + (ci & 1) * 32;
-    else
-      row0 = chh * 128 + ci * 32;
-    rd.w_ld[ci] = (row0 + lrow) * kBK;
-  }
-#pragma unroll
-  for (int tj = 0; tj < 2; ++tj) rd.x_ld[tj] = kTokOffset + (tb * 64 + tj * 32 + lrow) * kBK;
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk) rd.chunk[kk] = ((2 * kk + lhalf) ^ lsw) * 16;
 
@@ -453,53 +531,82 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(TileParams p) {
   while (tk.e == -2) tk = decode(it += stride);
   if (tk.e < 0) return;
   TaskLoads ld;
-  setup_loads<MODE>(p, tk, wave, lane, ld);
-  bool my_tokens = tb < tk.nsub;
-  int parity = 0;
+  setup_loads<MODE, DEEP>(p, tk, wave, lane, ld);
+  bool my_tokens = load_sub < tk.nsub;
+  int slot = 0;  // stage of the step being multiplied
   // The scratch of the tile list lived in the stage memory; everybody is past it (the builder ends
-  // with a barrier), so the first stage can be filled now.
-  issue_stage_loads(ld, p.a_q, stage0, wave, 0, my_tokens);
+  // with a barrier), so the first stage(s) can be filled now.
+  issue_stage_loads<DEEP>(ld, p.a_q, stage0, wave, 0, my_tokens);
+  if constexpr (DEEP) issue_stage_loads<DEEP>(ld, p.a_q, stage0 + kStageBytes, wave, kBK, my_tokens);
+  constexpr int kLoadsPerStep = 4 + G::kTokLoads;  // per wavefront (deep geometry: always that many)
 
   bool stores_pending = false;
   while (true) {
-    v16i acc[4][2];
-#pragma unroll
-    for (int ci = 0; ci < 4; ++ci)
-#pragma unroll
-      for (int tj = 0; tj < 2; ++tj)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[ci][tj][r] = 0;
-
-    // look ahead: the first loads of the next task are issued during the last step of this one
+    // look ahead: the first loads of the next task are issued during the last step(s) of this one
     int nit = it + stride;
     Task nx = decode(nit);
     while (nx.e == -2) nx = decode(nit += stride);
     TaskLoads nld = ld;
-    if (nx.e >= 0) setup_loads<MODE>(p, nx, wave, lane, nld);
-    const bool nx_tokens = tb < nx.nsub;
+    if (nx.e >= 0) setup_loads<MODE, DEEP>(p, nx, wave, lane, nld);
+    const bool nx_tokens = load_sub < nx.nsub;
 
-    for (int s = 0; s < nk; ++s) {
-      // this wavefront's loads of step s have landed (nothing newer is in flight) ...  A wavefront
-      // that has just run an epilogue waited for its loads there and only has the epilogue's
-      // stores pending: it lets them drain behind the first step instead of stalling on them.
-      if (s > 0 || !stores_pending) wait_vmcnt<0>();
-      // ... and so have everybody's; everybody is also done reading the other stage
+    // NCI = MFMA tiles of 32 weight rows per wavefront; `active`: the wavefront multiplies in this task
+    auto run_task = [&](auto nci_tag, bool active) {
+      constexpr int NCI = decltype(nci_tag)::value;
+      v16i acc[NCI][2];
+#pragma unroll
+      for (int ci = 0; ci < NCI; ++ci)
+#pragma unroll
+        for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[ci][tj][r] = 0;
+      make_reads<MODE, NCI>(wave, lane, rd);
+      for (int s = 0; s < nk; ++s) {
+        // This wavefront's loads of step s have landed ...  A wavefront that has just run an
+        // epilogue waited for all its loads there and only has the epilogue's stores pending: it
+        // lets them drain behind the first step instead of stalling on them.
+        if constexpr (DEEP) {
+          // in flight behind step s: the loads of step s + 1 (issued one step ago), if there is one
+          if (s > 0 || !stores_pending) {
+            if (s + 1 < nk || nx.e >= 0)
+              wait_vmcnt<kLoadsPerStep>();
+            else
+              wait_vmcnt<0>();
+          }
+        } else {
+          if (s > 0 || !stores_pending) wait_vmcnt<0>();
+        }
+        // ... and so have everybody's; everybody is also done reading the stage of the step before,
+        // which is the one to fill next
+        __builtin_amdgcn_s_barrier();
+        constexpr int kAhead = G::kSlots - 1;
+        int fill = slot + kAhead;
+        if (fill >= G::kSlots) fill -= G::kSlots;
+        const uint32_t fill_addr = stage0 + fill * kStageBytes;
+        if (s + kAhead < nk)
+          issue_stage_loads<DEEP>(ld, p.a_q, fill_addr, wave, (s + kAhead) * kBK, my_tokens);
+        else if (nx.e >= 0)
+          issue_stage_loads<DEEP>(nld, p.a_q, fill_addr, wave, (s + kAhead - nk) * kBK, nx_tokens);
+        if (active) multiply_stage<NCI>(rd, stages + slot * kStageBytes, acc);
+        slot = slot + 1 == G::kSlots ? 0 : slot + 1;
+      }
+      // everybody is done reading the stage of the last step: it becomes the epilogue's staging area
+      // (the next task's first loads went to the other stages)
       __builtin_amdgcn_s_barrier();
-      const uint32_t other = stage0 + (parity ^ 1) * kStageBytes;
-      if (s + 1 < nk)
-        issue_stage_loads(ld, p.a_q, other, wave, (s + 1) * kBK, my_tokens);
-      else if (nx.e >= 0)
-        issue_stage_loads(nld, p.a_q, other, wave, 0, nx_tokens);
-      if (my_tokens) multiply_stage(rd, stages + parity * kStageBytes, acc);
-      parity ^= 1;
+      const int last = slot == 0 ? G::kSlots - 1 : slot - 1;
+      if (active)
+        epilogue<MODE, NCI>(p, tk, wave, lane, acc, stages + last * kStageBytes + wave * 8192 / (4 / NCI),
+                            channel_scales + wave * 128);
+      stores_pending = active && MODE != kAccI32;
+    };
+    if constexpr (DEEP) {
+      if (tk.nsub >= 2)
+        run_task(std::integral_constant<int, 2>{}, true);
+      else
+        run_task(std::integral_constant<int, 1>{}, true);
+    } else {
+      run_task(std::integral_constant<int, 4>{}, load_sub < tk.nsub);
     }
-    // everybody is done reading the stage of the last step: it becomes the epilogue's staging area
-    // (the next task's first loads went to the other stage)
-    __builtin_amdgcn_s_barrier();
-    if (my_tokens)
-      epilogue<MODE>(p, tk, chh, tb, lane, acc, stages + (parity ^ 1) * kStageBytes + wave * 8192,
-                     channel_scales + wave * 128);
-    stores_pending = my_tokens && MODE != kAccI32;
     if (nx.e < 0) break;
     tk = nx;
     ld = nld;
@@ -509,7 +616,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(TileParams p) {
   wait_vmcnt<0>();
 }
 
-template <int MODE>
+template <int MODE, bool DEEP>
 hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   TileParams p;
   p.a_q = a.a_q;
@@ -529,33 +636,66 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   p.ntiles = MODE == kGateUpSilu ? (a.n / 2 + 127) / 128 : (a.n + kBN - 1) / kBN;
   p.out = a.out;
   const int grid = device_cu_count() / kXcds * kXcds;
-  hipLaunchKernelGGL(gemm_tile_kernel<MODE>, dim3((unsigned)grid), dim3(kThreads), 0, stream, p);
+  hipLaunchKernelGGL((gemm_tile_kernel<MODE, DEEP>), dim3((unsigned)grid), dim3(kThreads), 0, stream, p);
   return hipGetLastError();
 }
 
-}  // namespace
-
-bool gemm_tile_supports(const GemmArgs& a) {
+template <bool DEEP>
+bool geometry_supports(const GemmArgs& a) {
+  using G = Geometry<DEEP>;
   // per-lane source offsets are 32-bit: one expert's weights and the activation matrix must each
   // span less than 4 GiB
   const int64_t act_rows = (a.num_pairs + a.row_div - 1) / a.row_div;
-  if (!((a.block_size == 64 || a.block_size == 128) && a.k % kBK == 0 && a.k >= 2 * kBK && a.n % 16 == 0 &&
+  if (!((a.block_size == 64 || a.block_size == 128) && a.k % kBK == 0 && a.k >= G::kSlots * kBK && a.n % 16 == 0 &&
         (int64_t)a.n * a.k < (1ll << 32) && act_rows * a.k < (1ll << 32)))
     return false;
   // The tile list lives in LDS.  A run of equal expert ids of L blocks makes ceil(L / blocks per
   // tile) tiles; moe_align's ids ascend, so there is one run per expert.  Ids of unknown order could
   // make every block a tile of its own.  While the list is built the block ids sit in the stages.
   const int64_t blocks = (a.sorted_cap + a.block_size - 1) / a.block_size;
-  const int per_tile = kTileTok / a.block_size;
+  const int per_tile = G::kTileTok / a.block_size;
   const int64_t tiles = a.expert_ids_ascend ? (blocks + per_tile - 1) / per_tile + a.num_experts : blocks;
-  return tiles <= kMaxTiles && blocks <= (int64_t)(2 * kStageBytes / sizeof(int)) && blocks <= 65535;
+  return tiles <= G::kMaxTiles && blocks <= (int64_t)(G::kSlots * G::kStageBytes / sizeof(int)) && blocks <= 65535;
+}
+
+}  // namespace
+
+bool gemm_tile_supports(const GemmArgs& a) {
+  switch (a.tile_geometry) {
+    case kTileWide: return geometry_supports<false>(a);
+    case kTileDeep: return geometry_supports<true>(a);
+    default: return geometry_supports<false>(a) || geometry_supports<true>(a);
+  }
+}
+
+// Measured on three layer shapes (Qwen3-30B-A3B, GLM-4.5-Air, DeepSeek-V3): the deep geometry wins up
+// to about a hundred routed rows per expert, where a 256-row tile would be mostly padding and the
+// kernel is bound by the weight stream; beyond that the wide tile's reuse of a weight tile by up to
+// four sub-blocks wins.
+bool gemm_tile_prefers_deep(const GemmArgs& a) {
+  return a.num_pairs <= (int64_t)kTileDeepRowsPerExpert * a.num_experts;
 }
 
 hipError_t launch_gemm_tile(const GemmArgs& a, hipStream_t stream) {
+  bool deep;
+  if (a.tile_geometry == kTileWide)
+    deep = false;
+  else if (a.tile_geometry == kTileDeep)
+    deep = true;
+  else
+    deep = geometry_supports<true>(a) && (gemm_tile_prefers_deep(a) || !geometry_supports<false>(a));
+  if (deep) {
+    switch (a.mode) {
+      case kGateUpSilu: return launch_mode<kGateUpSilu, true>(a, stream);
+      case kDown: return launch_mode<kDown, true>(a, stream);
+      case kAccI32: return launch_mode<kAccI32, true>(a, stream);
+      default: return hipErrorInvalidValue;
+    }
+  }
   switch (a.mode) {
-    case kGateUpSilu: return launch_mode<kGateUpSilu>(a, stream);
-    case kDown: return launch_mode<kDown>(a, stream);
-    case kAccI32: return launch_mode<kAccI32>(a, stream);
+    case kGateUpSilu: return launch_mode<kGateUpSilu, false>(a, stream);
+    case kDown: return launch_mode<kDown, false>(a, stream);
+    case kAccI32: return launch_mode<kAccI32, false>(a, stream);
     default: return hipErrorInvalidValue;
   }
 }

@@ -37,7 +37,7 @@ def _check_against_oracle(pra, oracle, shape_name, M, seed, variant="auto"):
 @pytest.mark.parametrize("variant", ["stream", "auto"])
 @pytest.mark.parametrize("shape_name,M", [
     ("toy", 256), ("toy", 1), ("qwen3-30b-a3b", 16), ("qwen3-30b-a3b", 128), ("qwen3-30b-a3b", 1024),
-    ("glm-4.5-air", 32),
+    ("qwen3-30b-a3b", 2048), ("glm-4.5-air", 32),
 ])
 def test_fused_experts_matches_oracle(pra, oracle, shape_name, M, variant):
     _check_against_oracle(pra, oracle, shape_name, M, seed=M, variant=variant)
@@ -115,7 +115,7 @@ def test_block_size_does_not_change_the_result(pra):
         assert torch.equal(ref, _run(pra, inp, block_size_m=B))
 
 
-@pytest.mark.parametrize("M", [16, 512, 2048])  # streaming, narrow-tile and wide-tile GEMM families
+@pytest.mark.parametrize("M", [16, 512, 1024, 2048])  # streaming, narrow-tile, deep and wide LDS-tile GEMM families
 def test_hip_graph_replay(pra, M):
     """The call records no allocation, memset or synchronisation, so it can be captured and replayed."""
     im = inputs_mod()
@@ -214,11 +214,14 @@ FULL_SIZE = [
 def test_full_size_whole_output_equal_across_families(pra, shape_name, M):
     im = inputs_mod()
     inp = im.make_inputs(shape_name, M, seed=M + 7, device=DEV, weights_on_device=True)
-    auto = _run(pra, inp, gemm_variant="auto")
     stream = _run(pra, inp, gemm_variant="stream")
-    assert bool(torch.isfinite(auto.float()).all())
-    differing = int((auto != stream).sum())
-    assert differing == 0, f"{differing} of {auto.numel()} elements differ between the families"
+    assert bool(torch.isfinite(stream.float()).all())
+    # what the library picks by itself, and both geometries of the LDS-tiled family
+    for variant in ("auto", "tile_wide", "tile_deep"):
+        tiled = _run(pra, inp, gemm_variant=variant)
+        differing = int((tiled != stream).sum())
+        assert differing == 0, f"{variant}: {differing} of {tiled.numel()} elements differ between the families"
+        del tiled
     # and stage by stage on the device: the down GEMM of the tiled family against the streaming one
     P = M * inp.topk_ids.shape[1]
     x_q, a1 = pra.per_token_quant_int8(inp.hidden_states)
