@@ -60,13 +60,13 @@ int tile_geometry_of(int variant) {
 
 // Routed rows per expert up to which the narrow tiles beat the deep geometry of the LDS-tiled family.
 // The narrow tiles (two small workgroups per compute unit, 64 x 128 tasks) start up faster and
-// balance better; the deep tiles stream an expert's weights once for up to 128 rows and sustain
-// more bytes in flight, which counts the more the longer a launch runs.  Measured crossovers, with
-// the weight bytes of the launch: 0.2-0.4 GB (Qwen3-30B-A3B) 44-48 rows, 0.7-1.5 GB (GLM-4.5-Air)
-// 22-30, 3.8-7.5 GB (DeepSeek-V3) at most 8.
+// balance better; the deep tiles stream an expert's weights once for up to 128 rows, which counts
+// the more the longer a launch runs and the more the routing is skewed.  Measured crossovers, with
+// the weight bytes of the launch: 0.2-0.4 GB (Qwen3-30B-A3B, even routing) 32-48 rows, 0.7-1.5 GB
+// (GLM-4.5-Air, Zipf routing and a shared expert) 24-32, 3.8-7.5 GB (DeepSeek-V3) below 8.
 int narrow_rows_per_expert(const moe_i8::GemmArgs& g) {
   const int64_t weight_bytes = (int64_t)g.num_experts * g.n * g.k;
-  return weight_bytes < (512ll << 20) ? 48 : weight_bytes < (2048ll << 20) ? 24 : 12;
+  return weight_bytes < (512ll << 20) ? 44 : weight_bytes < (2048ll << 20) ? 24 : 8;
 }
 
 // Which family a launch goes to (MOE_I8_GEMM_STREAM, _TILE or _NARROW); -1 with the error set if a
