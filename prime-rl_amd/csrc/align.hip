@@ -1,10 +1,11 @@
 // moe_align_block_size for gfx950: stable counting sort of (token, expert) pairs by expert,
 // each expert segment padded to a multiple of the block size.
 //
-// The unit of work is one 64-lane wavefront walking a contiguous chunk of pairs.  Inside a
-// wavefront the rank of a pair among the lanes that hold the same expert comes from ballots
-// (one per bit of the expert id) and a population count below the lane, so no atomics are
-// needed and the order inside an expert segment is the ascending flat pair index.
+// The unit of work is one 64-lane wavefront walking a contiguous chunk of pairs.  Counting uses
+// LDS atomics on counters private to the wavefront (a count has no order).  In the scatter the
+// rank of a pair among the lanes that hold the same expert comes from ballots (one per bit of the
+// expert id) and a population count below the lane, so the order inside an expert segment is the
+// ascending flat pair index whatever order the hardware resolves conflicts in.
 //
 // Small inputs run in one 1024-thread workgroup (histogram, scans and scatter fused).  Large
 // inputs use three launches: per-wave histograms, one scan workgroup, scatter.
@@ -47,20 +48,16 @@ __device__ __forceinline__ void wave_load_ids(const int32_t* __restrict__ ids, i
   }
 }
 
-// counts[x] += number of loaded pairs routed to x; counts is private to the wavefront.
+// counts[x] += number of loaded pairs routed to x; counts is private to the wavefront (LDS).  Counting
+// needs no order, so it is one LDS atomic per pair (lanes that hit the same counter are serialised by
+// the LDS); only the scatter below needs the rank of a pair among its peers.
 template <int kIters>
-__device__ __forceinline__ void wave_histogram(const int (&ids)[kIters], int64_t count, int E, int nbits,
-                                               int* counts) {
-  const int lane = lane_id();
+__device__ __forceinline__ void wave_histogram(const int (&ids)[kIters], int64_t count, int E, int* counts) {
 #pragma unroll
   for (int i = 0; i < kIters; ++i) {
     if ((int64_t)i * kWave >= count) break;  // wave-uniform: nothing left in this wavefront's range
     const int e = ids[i];
-    const bool active = e >= 0 && e < E;
-    const uint64_t peers = peers_of(e, active, nbits);
-    const int rank = __popcll(peers & ((1ull << lane) - 1ull));
-    if (active && rank == 0) counts[e] += __popcll(peers);
-    __builtin_amdgcn_wave_barrier();
+    if (e >= 0 && e < E) atomicAdd(counts + e, 1);
   }
 }
 
@@ -154,7 +151,7 @@ __device__ __forceinline__ void align_single_body(
   const int64_t end = begin + per_wave < P ? begin + per_wave : P;
   int mine[kSingleIters];
   wave_load_ids(ids, begin, end, mine);
-  wave_histogram(mine, end - begin, E, nbits, hist + wave * E);
+  wave_histogram(mine, end - begin, E, hist + wave * E);
   __syncthreads();
 
   int padded = 0;
@@ -212,16 +209,16 @@ __global__ __launch_bounds__(kSingleThreads) void align_quant_kernel(
 
 // smem[w][e] = number of pairs of wavefront w's quarter routed to e
 __device__ __forceinline__ void unit_wave_histograms(const int (&mine)[kMultiIters], int64_t count, int E,
-                                                     int nbits, int* smem) {
+                                                     int* smem) {
   const int tid = threadIdx.x;
   for (int i = tid; i < kMultiWaves * E; i += kMultiThreads) smem[i] = 0;
   __syncthreads();
-  wave_histogram(mine, count, E, nbits, smem + (tid / kWave) * E);
+  wave_histogram(mine, count, E, smem + (tid / kWave) * E);
   __syncthreads();
 }
 
 __global__ __launch_bounds__(kMultiThreads) void align_hist_kernel(
-    const int32_t* __restrict__ ids, int64_t P, int E, int nbits, int32_t* __restrict__ unit_hist,
+    const int32_t* __restrict__ ids, int64_t P, int E, int32_t* __restrict__ unit_hist,
     int32_t* __restrict__ sorted, int64_t sorted_cap) {
   extern __shared__ int smem[];
   const int tid = threadIdx.x;
@@ -232,7 +229,7 @@ __global__ __launch_bounds__(kMultiThreads) void align_hist_kernel(
   for (int64_t i = (int64_t)blockIdx.x * kMultiThreads + tid; i < sorted_cap;
        i += (int64_t)gridDim.x * kMultiThreads)
     sorted[i] = (int32_t)P;
-  unit_wave_histograms(mine, end - begin, E, nbits, smem);
+  unit_wave_histograms(mine, end - begin, E, smem);
   for (int e = tid; e < E; e += kMultiThreads) {
     int sum = 0;
 #pragma unroll
@@ -305,7 +302,7 @@ __global__ __launch_bounds__(kMultiThreads) void align_scatter_kernel(
   const int64_t end = begin + kMultiChunk / kMultiWaves < P ? begin + kMultiChunk / kMultiWaves : P;
   int mine[kMultiIters];
   wave_load_ids(ids, begin, end, mine);
-  unit_wave_histograms(mine, end - begin, E, nbits, smem);
+  unit_wave_histograms(mine, end - begin, E, smem);
   // counts -> write cursors: segment start + pairs of earlier units + pairs of earlier wavefronts
   for (int e = tid; e < E; e += kMultiThreads) {
     int run = seg[e] + unit_base[(int64_t)blockIdx.x * E + e];
@@ -356,7 +353,7 @@ hipError_t launch_align_quant(const AlignArgs& a, const QuantArgs& q, hipStream_
     int32_t* seg = unit_base + (int64_t)units * E;
     const size_t lds = sizeof(int) * (size_t)kMultiWaves * E;
     hipLaunchKernelGGL(align_hist_kernel, dim3(units), dim3(kMultiThreads), lds, stream, a.topk_ids,
-                       a.num_pairs, E, nbits, unit_hist, a.sorted_token_ids, a.sorted_cap);
+                       a.num_pairs, E, unit_hist, a.sorted_token_ids, a.sorted_cap);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
 #define MOE_I8_SCAN_QUANT(V)                                                                           \
@@ -421,7 +418,7 @@ hipError_t launch_align(const AlignArgs& a, hipStream_t stream) {
   int32_t* seg = unit_base + (int64_t)units * E;
   const size_t lds = sizeof(int) * (size_t)kMultiWaves * E;
   hipLaunchKernelGGL(align_hist_kernel, dim3(units), dim3(kMultiThreads), lds, stream, a.topk_ids,
-                     a.num_pairs, E, nbits, unit_hist, a.sorted_token_ids, a.sorted_cap);
+                     a.num_pairs, E, unit_hist, a.sorted_token_ids, a.sorted_cap);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return err;
   hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kSingleThreads), 0, stream, E, a.block_size,
