@@ -513,7 +513,8 @@ def cpu_baseline(oracle, torch, base, sample_m: int) -> dict:
             base.w1_scale, base.w2_scale)
     oracle.native_w8a8_moe(*args)  # warm-up
     best = float("inf")
-    for _ in range(2):
+    passes = 5
+    for _ in range(passes):
         t0 = time.perf_counter()
         oracle.native_w8a8_moe(*args)
         best = min(best, time.perf_counter() - t0)
@@ -523,7 +524,7 @@ def cpu_baseline(oracle, torch, base, sample_m: int) -> dict:
         "cores": torch.get_num_threads(),
         "kind": "port",
         "sample": f"first {m} tokens of the same seeded workload, torch-native W8A8 MoE of the oracle, "
-                  f"best of 2 after 1 warm-up ({best:.2f} s per pass; os.cpu_count()={os.cpu_count()})",
+                  f"best of {passes} after 1 warm-up ({best:.2f} s per pass; os.cpu_count()={os.cpu_count()})",
     }
 
 
@@ -542,7 +543,7 @@ def main() -> int:
     ap.add_argument("--no-other-shapes", action="store_true")
     ap.add_argument("--decode-layers", type=int, default=48)
     ap.add_argument("--decode-steps", type=int, default=500)
-    ap.add_argument("--cpu-sample", type=int, default=4096, help="tokens of the workload the CPU baseline runs")
+    ap.add_argument("--cpu-sample", type=int, default=8192, help="tokens of the workload the CPU baseline runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
