@@ -83,15 +83,7 @@ __device__ __forceinline__ void wave_scatter(const int (&ids)[kIters], int64_t b
   }
 }
 
-__device__ __forceinline__ int wave_inclusive_scan(int v) {
-  const int lane = lane_id();
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    const int n = __shfl_up(v, d);
-    if (lane >= d) v += n;
-  }
-  return v;
-}
+__device__ __forceinline__ int wave_inclusive_scan(int v) { return wave_inclusive_scan_add(v); }
 
 // Exclusive scan over the 1024 threads of the block; returns the exclusive prefix, *total = sum.
 __device__ __forceinline__ int block_exclusive_scan_1024(int v, int* wave_sums, int* total) {

@@ -72,6 +72,7 @@ struct TileParams {
   int K;
   int B;
   int ntiles;  // channel tiles
+  int ascend;  // expert_ids is known to ascend over the used blocks (it comes from moe_align)
   void* out;
 };
 
@@ -182,6 +183,69 @@ __device__ int build_tile_list(const int32_t* __restrict__ expert_ids, int nbloc
   }
   __syncthreads();
   return total;
+}
+
+// The same list when the expert ids are known to ascend over the used blocks (what moe_align writes):
+// every expert then owns at most one run of blocks, found by comparing a block with its neighbours, and
+// the number of tiles in front of an expert is one scan over the experts instead of two over the blocks
+// (a third of the time on a long list).  Runs of ids outside [0, E) get no tiles.  scratch holds
+// 2 * num_experts ints; per_tile is 1 << per_tile_log2.
+__device__ int build_tile_list_ascending(const int32_t* __restrict__ expert_ids, int nblocks, int num_experts,
+                                         int per_tile_log2, int* scratch, int* wave_part, uint32_t* tile_desc,
+                                         int* total_out, int max_tiles) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  int* first = scratch;               // first block of the expert's run
+  int* end = scratch + num_experts;   // one past its last block
+  for (int e = tid; e < 2 * num_experts; e += kThreads) scratch[e] = 0;
+  __syncthreads();
+  for (int j = tid; j < nblocks; j += kThreads) {
+    const int e = expert_ids[j];
+    const int prev = j > 0 ? expert_ids[j - 1] : -1;
+    const int next = j + 1 < nblocks ? expert_ids[j + 1] : -1;
+    if (e >= 0 && e < num_experts) {
+      if (j == 0 || e != prev) first[e] = j;
+      if (j + 1 == nblocks || e != next) end[e] = j + 1;
+    }
+  }
+  __syncthreads();
+  // thread t owns experts 2t and 2t + 1 (num_experts <= 2 * kThreads)
+  const int per_tile = 1 << per_tile_log2;
+  int f[2], nb[2], tiles[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int e = 2 * tid + i;
+    f[i] = e < num_experts ? first[e] : 0;
+    nb[i] = e < num_experts ? end[e] - f[i] : 0;
+    tiles[i] = (nb[i] + per_tile - 1) >> per_tile_log2;
+  }
+  const int mine = tiles[0] + tiles[1];
+  const int incl = wave_inclusive_scan_add(mine);
+  if (lane == kWave - 1) wave_part[wave] = incl;
+  __syncthreads();
+  int carry = 0, total = 0;
+#pragma unroll
+  for (int i = 0; i < kWaves; ++i) {
+    const int w = wave_part[i];
+    if (i < wave) carry += w;
+    total += w;
+  }
+  int t = carry + incl - mine;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    for (int r = 0; r < tiles[i]; ++r, ++t) {
+      if (t >= max_tiles) break;
+      const int left = nb[i] - (r << per_tile_log2);
+      const int in_group = tiles[i] - (r & ~(kGroupTiles - 1));
+      tile_desc[t] = (uint32_t)(f[i] + (r << per_tile_log2)) | ((uint32_t)(left < per_tile ? left : per_tile) << 16) |
+                     ((uint32_t)(r & (kGroupTiles - 1)) << 20) |
+                     ((uint32_t)(in_group < kGroupTiles ? in_group : kGroupTiles) << 24);
+    }
+  }
+  if (tid == 0) *total_out = total < max_tiles ? total : max_tiles;
+  __syncthreads();
+  return total < max_tiles ? total : max_tiles;
 }
 
 struct Task {
@@ -484,8 +548,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(TileParams p) {
   const int npp = *p.npp;
   const int nblocks = npp / p.B;
   const int sub_per_block = p.B / 64;
-  const int ntile = build_tile_list(p.expert_ids, nblocks, G::kTileTok / p.B, reinterpret_cast<int*>(stages),
-                                    wave_part, tile_desc, &total_tiles, G::kMaxTiles);
+  const int per_tile = G::kTileTok / p.B;  // 1, 2 or 4 blocks
+  const int ntile =
+      p.ascend ? build_tile_list_ascending(p.expert_ids, nblocks, p.E, per_tile == 4 ? 2 : per_tile == 2 ? 1 : 0,
+                                           reinterpret_cast<int*>(stages), wave_part, tile_desc, &total_tiles,
+                                           G::kMaxTiles)
+               : build_tile_list(p.expert_ids, nblocks, per_tile, reinterpret_cast<int*>(stages), wave_part, tile_desc,
+                                 &total_tiles, G::kMaxTiles);
   const int total = ntile * p.ntiles;
   const int per_xcd = (total + kXcds - 1) / kXcds;
   const int xcd = blockIdx.x % kXcds;
@@ -634,6 +703,7 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   p.K = a.k;
   p.B = a.block_size;
   p.ntiles = MODE == kGateUpSilu ? (a.n / 2 + 127) / 128 : (a.n + kBN - 1) / kBN;
+  p.ascend = a.expert_ids_ascend && a.num_experts <= 2 * kThreads ? 1 : 0;
   p.out = a.out;
   const int grid = device_cu_count() / kXcds * kXcds;
   hipLaunchKernelGGL((gemm_tile_kernel<MODE, DEEP>), dim3((unsigned)grid), dim3(kThreads), 0, stream, p);
