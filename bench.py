@@ -118,7 +118,10 @@ def time_gate_up_kernel(pkg, torch, shape, dev, weights, steps: int, warmup: int
 def time_stages(pkg, torch, shape, dev, weights, steps: int, warmup: int, variant: str) -> list:
     """Every launch of the layer on its own: direct C-ABI calls into preallocated buffers, an event pair per
     call on the launch stream, with the algorithmic bytes / int8 ops of that launch and the fraction of the
-    roofline that bounds it.  (A launch that does almost nothing still reads about 4 us.)"""
+    roofline that bounds it.  (A launch that does almost nothing still reads about 4 us.  Timed alone back to
+    back the gate_up GEMM reads about 10 % above its duration inside the layer, where the memory-bound
+    launches around it let the clock recover; the dispatch durations of a kernel trace of the whole layer are
+    the in-situ figures.)"""
     abi = pkg._abi
     lib = abi.load()
     M, k = dev.topk_ids.shape
