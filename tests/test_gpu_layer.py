@@ -262,3 +262,29 @@ def test_capture_never_allocates_the_default_workspace(pra):
             # eager work at the reserved size on the same stream between replays: same buffer, no regrowth
             pra.fused_experts(*big.fused_experts_args(), **big.fused_experts_kwargs())
             torch.cuda.synchronize()
+
+
+# The LDS-tiled family builds its tile list inside the kernel; inside fused_experts (expert ids known to
+# ascend) from per-expert runs, two experts per thread.  Routings that stress that list: more than 512
+# experts with most of them absent, a single expert holding every row (dozens of tiles of one expert,
+# i.e. several groups of eight), one row per expert, and both block sizes.  The streaming family has no
+# tile list, so bit-equality of the complete outputs is the check.
+@pytest.mark.parametrize("E,k,M,B,routing", [
+    (640, 2, 700, 64, "softmax"),     # > 512 experts: both slots of a thread, many absent experts
+    (1024, 1, 300, 64, "softmax"),    # the largest expert count the library takes, most experts absent
+    (8, 1, 3000, 64, "one_hot"),      # one expert holds all 3000 rows
+    (8, 1, 3000, 128, "one_hot"),
+    (40, 4, 10, 128, "softmax"),      # one row per expert at most
+    (16, 2, 1100, 128, "zipf"),
+])
+@pytest.mark.parametrize("variant", ["tile_wide", "tile_deep"])
+def test_tile_list_edge_routings(pra, E, k, M, B, routing, variant):
+    im = inputs_mod()
+    shape = im.LayerShape("edge", E=E, k=k, H=512, I=512, routing="softmax" if routing == "one_hot" else routing)
+    inp = im.make_inputs(shape, M, seed=E + M).to(DEV)
+    if routing == "one_hot":
+        inp.topk_ids.fill_(3)
+    want = _run(pra, inp, gemm_variant="stream", block_size_m=B)
+    got = _run(pra, inp, gemm_variant=variant, block_size_m=B)
+    differing = int((got != want).sum())
+    assert differing == 0, f"{differing} of {got.numel()} elements differ"
