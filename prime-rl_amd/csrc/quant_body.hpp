@@ -146,19 +146,46 @@ __device__ __forceinline__ void quant_one_row(const QuantArgs& a, int64_t row) {
       }
     }
   } else {
+    // four independent 16-byte loads per lane and trip, so that a long row is not one load latency per
+    // 1 KB of it
+    constexpr int kUnroll = 4;
     float m = 0.0f;
-    if (have)
-      for (int c = lane; c < nvec; c += kWave) m = fmaxf(m, absmax8(in[c]));
+    if (have) {
+      for (int c0 = lane; c0 < nvec; c0 += kUnroll * kWave) {
+        uint4 t[kUnroll];
+#pragma unroll
+        for (int i = 0; i < kUnroll; ++i) {
+          const int c = c0 + i * kWave;
+          t[i] = c < nvec ? in[c] : make_uint4(0u, 0u, 0u, 0u);
+        }
+#pragma unroll
+        for (int i = 0; i < kUnroll; ++i) m = fmaxf(m, absmax8(t[i]));
+      }
+    }
+    auto second_pass = [&](auto quantise) {
+      for (int c0 = lane; c0 < nvec; c0 += kUnroll * kWave) {
+        uint4 t[kUnroll];
+#pragma unroll
+        for (int i = 0; i < kUnroll; ++i) {
+          const int c = c0 + i * kWave;
+          t[i] = (have && c < nvec) ? in[c] : make_uint4(0u, 0u, 0u, 0u);
+        }
+#pragma unroll
+        for (int i = 0; i < kUnroll; ++i) {
+          const int c = c0 + i * kWave;
+          if (c < nvec) out[c] = have ? quantise(t[i]) : make_uint2(0u, 0u);
+        }
+      }
+    };
     if constexpr (kMode == kQuantWeights) {
       const WeightRcp s = weight_rcp(fmaxf(wave_max(m) / 127.0f, 1e-12f));
       if (lane == 0) a.scale[orow] = s.scale;
-      for (int c = lane; c < nvec; c += kWave) out[c] = have ? quant8_weights(in[c], s) : make_uint2(0u, 0u);
+      second_pass([&](const uint4& v) { return quant8_weights(v, s); });
     } else {
       const float absmax = fmaxf(wave_max(m), 1e-10f);
       const float inv = 127.0f / absmax;
       if (lane == 0) a.scale[orow] = absmax / 127.0f;
-      for (int c = lane; c < nvec; c += kWave)
-        out[c] = have ? quant8<kMode == kQuantEven>(in[c], inv) : make_uint2(0u, 0u);
+      second_pass([&](const uint4& v) { return quant8<kMode == kQuantEven>(v, inv); });
     }
   }
 }
