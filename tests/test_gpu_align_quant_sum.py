@@ -49,7 +49,8 @@ def test_align_baseline_routings(pra, oracle, shape_name, M):
 
 
 @pytest.mark.parametrize("B", [16, 32, 64, 128])
-@pytest.mark.parametrize("E,P", [(1, 1), (1, 700), (3, 2), (8, 8191), (8, 8193), (257, 9000), (1024, 5000), (1024, 70000)])
+@pytest.mark.parametrize("E,P", [(1, 1), (1, 700), (3, 2), (8, 8191), (8, 8193), (257, 9000), (1024, 5000), (1024, 70000),
+                                 (1024, 20000), (128, 32768), (128, 32769), (5, 12345)])  # the two- and three-launch paths
 def test_align_block_sizes_and_extremes(pra, oracle, B, E, P):
     ids = torch.randint(0, E, (P, 1), generator=torch.Generator().manual_seed(P + E), dtype=torch.int32)
     _check_align(pra, oracle, ids, B, E)
