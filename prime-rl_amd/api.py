@@ -52,10 +52,13 @@ _VARIANTS = {
 }
 # Default workspaces, one per (device, stream) that has called without a caller-owned one: a small
 # LRU (a process has a handful of forward streams) guarded by a lock.  Entries are only ever created or
-# grown outside HIP graph capture, so a captured graph never holds a pointer that a later call frees:
-# a capture that finds no entry large enough raises instead of allocating.
+# grown outside HIP graph capture (a capture that finds no entry large enough raises instead of
+# allocating), and an entry that a capture used or reserve_workspace made is never freed: when it is
+# outgrown it is retired to a keep-alive list, and eviction skips it.
 _MAX_CACHED_WORKSPACES = 16
 _workspaces: "OrderedDict[tuple[int, int], torch.Tensor]" = OrderedDict()
+_pinned_workspaces: "set[tuple[int, int]]" = set()  # keys whose buffer a capture or reserve_workspace handed out
+_retired_workspaces: "list[torch.Tensor]" = []      # outgrown pinned buffers, kept allocated
 _workspaces_lock = threading.Lock()
 
 
@@ -724,24 +727,40 @@ def _capturing(device: torch.device) -> bool:
     return bool(torch.cuda.is_available() and torch.cuda.is_current_stream_capturing())
 
 
-def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
+def _workspace(device: torch.device, stream: int, nbytes: int, pin: bool = False) -> torch.Tensor:
+    """Default workspace of a (device, stream).  A buffer that ``reserve_workspace`` allocated, or that a
+    call made under graph capture used, is *pinned*: a captured graph may hold its address, so it is never
+    replaced in place or evicted; when a later eager call needs more, the pinned buffer moves to a keep-alive
+    list (it stays allocated for the life of the process) and a larger one takes its place in the cache.
+    Only buffers that no capture has seen are freed, when the cache is over its size or they are outgrown."""
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
     with _workspaces_lock:
         ws = _workspaces.get(key)
+        capturing = _capturing(device)
         if ws is not None and ws.numel() >= nbytes:
             _workspaces.move_to_end(key)
+            if pin or capturing:
+                _pinned_workspaces.add(key)
             return ws
-        if _capturing(device):
+        if capturing:
             raise RuntimeError(
                 f"this call needs a {nbytes}-byte workspace while the stream is being captured into a graph and "
                 "none of that size was allocated for it beforehand: pass workspace=, or call reserve_workspace() "
                 "(or run the largest batch once eagerly on this stream) before capturing"
             )
+        if ws is not None and key in _pinned_workspaces:
+            _retired_workspaces.append(ws)  # a graph may replay on it: keep it allocated
+            _pinned_workspaces.discard(key)
         ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
         _workspaces.move_to_end(key)
-        while len(_workspaces) > _MAX_CACHED_WORKSPACES:
-            _workspaces.popitem(last=False)
+        if pin:
+            _pinned_workspaces.add(key)
+        if len(_workspaces) > _MAX_CACHED_WORKSPACES:
+            for old_key in [k for k in _workspaces if k not in _pinned_workspaces and k != key]:
+                if len(_workspaces) <= _MAX_CACHED_WORKSPACES:
+                    break
+                del _workspaces[old_key]
         return ws
 
 
@@ -749,10 +768,12 @@ def reserve_workspace(max_tokens: int, top_k: int, num_experts: int, hidden: int
                       block_size_m: int = DEFAULT_BLOCK_SIZE_M) -> torch.Tensor:
     """Allocate now (outside any graph capture) the default workspace that ``fused_experts`` calls on the
     current stream of ``device`` use for up to ``max_tokens`` tokens of this layer shape, so that captured
-    calls find it.  The tensor stays cached for that (device, stream); it is also returned."""
+    calls find it.  The tensor stays allocated for the life of the process (graphs captured against it stay
+    valid whatever later calls need); it is also returned."""
     device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
     stream = torch.cuda.current_stream(device).cuda_stream
-    return _workspace(device, stream, workspace_bytes(max_tokens, top_k, num_experts, hidden, inter, block_size_m))
+    return _workspace(device, stream, workspace_bytes(max_tokens, top_k, num_experts, hidden, inter, block_size_m),
+                      pin=True)
 
 
 def fused_experts(

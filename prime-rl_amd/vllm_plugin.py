@@ -12,8 +12,10 @@ Two surfaces are covered:
 
 * the flat ``fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, ..., use_int8_w8a8=True, ...)``
   function: calls this library handles go to the HIP path, everything else (another quantisation
-  mode, an expert map, a keyword this library does not know, a shape it rejects) falls through to
-  the original;
+  mode, an expert map, a bias, a keyword this library does not know, a shape it rejects — decided from
+  the shapes before the call, and again if the entry's own validation raises ``ValueError`` or
+  ``NotImplementedError``) falls through to the original.  Errors raised while the HIP path runs
+  (a failed launch, a capture without a reserved workspace) are not swallowed;
 * the modular-kernel surface the pinned vLLM selects kernels through (``FusedMoE`` is a factory
   returning a ``MoERunner``, reference ``src/prime_rl/inference/vllm/worker/weight_transfer.py:76-82``;
   the choice of experts implementation goes through ``FusedMoEConfig``, ``patches.py:740-757``):
@@ -54,31 +56,68 @@ def _accepted_keywords(fn) -> frozenset:
     )
 
 
-def _handles(hidden_states, kwargs, accepted) -> bool:
-    if not kwargs.get("use_int8_w8a8", False) or not kwargs.get("per_channel_quant", False):
+def _present(value) -> bool:
+    """A keyword counts as set unless it is None or False.  Decided by identity only: the value may be a
+    tensor (an expert map, a bias, zero points), whose truth value is ambiguous or forces a device sync."""
+    return value is not None and value is not False
+
+
+def _shapes_eligible(hidden_states, w1, w2, kwargs) -> bool:
+    """The argument checks of the HIP entry that depend on shapes only, made up front so that a layer this
+    library cannot take goes to the original instead of failing the forward pass.  Objects without shapes
+    (nothing to check) pass; the entry validates again."""
+    try:
+        s1, s2, sx = tuple(w1.shape), tuple(w2.shape), tuple(hidden_states.shape)
+    except (AttributeError, TypeError):
+        return True
+    if len(sx) != 2 or len(s1) != 3 or len(s2) != 3:
+        return False
+    experts, n1, hidden = s1
+    if n1 % 2 or sx[1] != hidden or s2 != (experts, hidden, n1 // 2):
+        return False
+    if experts > 1024 or hidden % 64 or (n1 // 2) % 64:
+        return False
+    gne = kwargs.get("global_num_experts", -1)
+    return gne in (-1, experts)
+
+
+def _handles(hidden_states, w1, w2, kwargs, accepted) -> bool:
+    if kwargs.get("use_int8_w8a8", False) is not True or kwargs.get("per_channel_quant", False) is not True:
         return False
     if kwargs.get("activation", "silu") != "silu":
         return False
-    if any(kwargs.get(flag) for flag in _OTHER_MODE_FLAGS):
+    if any(_present(kwargs.get(flag)) for flag in _OTHER_MODE_FLAGS):
         return False
     # a keyword this library has never heard of may change the meaning of the call
-    if any(k not in accepted and k not in _OTHER_MODE_FLAGS and v not in (None, False) for k, v in kwargs.items()):
+    if any(k not in accepted and k not in _OTHER_MODE_FLAGS and _present(v) for k, v in kwargs.items()):
         return False
-    return bool(getattr(hidden_states, "is_cuda", False)) and str(getattr(hidden_states, "dtype", "")) == "torch.bfloat16"
+    if kwargs.get("w1_scale") is None or kwargs.get("w2_scale") is None:
+        return False
+    if not (bool(getattr(hidden_states, "is_cuda", False)) and str(getattr(hidden_states, "dtype", "")) == "torch.bfloat16"):
+        return False
+    return _shapes_eligible(hidden_states, w1, w2, kwargs)
 
 
 def _wrap(original, hip_fused_experts=None):
     if hip_fused_experts is None:
         from .api import fused_experts as hip_fused_experts
     accepted = _accepted_keywords(hip_fused_experts)
+    signature = inspect.signature(hip_fused_experts)
 
     def fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, *args, **kwargs):
-        if not args and _handles(hidden_states, kwargs, accepted):
+        if not args and _handles(hidden_states, w1, w2, kwargs, accepted):
             forwarded = {k: v for k, v in kwargs.items() if k in accepted}
             try:
-                return hip_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, **forwarded)
-            except (NotImplementedError, TypeError):
-                pass  # a mode or shape this library rejects: the original handles it
+                signature.bind(hidden_states, w1, w2, topk_weights, topk_ids, **forwarded)
+            except TypeError:
+                bound = False  # the call does not fit the HIP entry's signature: not ours
+            else:
+                bound = True
+            if bound:
+                try:
+                    return hip_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, **forwarded)
+                except (NotImplementedError, ValueError):
+                    pass  # a mode or shape the entry's own validation rejects: the original handles it
         return original(hidden_states, w1, w2, topk_weights, topk_ids, *args, **kwargs)
 
     setattr(fused_experts, _MARK, True)

@@ -47,8 +47,13 @@ def plugin(pra, monkeypatch):
                           global_num_experts=-1, expert_map=None, w1_scale=None, w2_scale=None, a1_scale=None,
                           a2_scale=None, block_shape=None, *, workspace=None):
         hip_calls.append(dict(use_int8_w8a8=use_int8_w8a8, w1_scale=w1_scale, global_num_experts=global_num_experts))
-        if w1_scale == "unsupported-shape":
+        tag = w1_scale if isinstance(w1_scale, str) else ""
+        if tag == "unsupported-shape":
             raise NotImplementedError("shape")
+        if tag == "rejected-by-validation":
+            raise ValueError("w2 must be [E, H, I]")
+        if tag == "launch-failed":
+            raise RuntimeError("launch")
         return "hip"
 
     monkeypatch.setattr(pra.api, "fused_experts", hip_fused_experts)
@@ -111,6 +116,74 @@ def test_dispatch_and_fall_through(plugin, monkeypatch):
     assert fe(x, 1, 2, 3, 4, **{**int8, "w1_scale": "unsupported-shape"}) == "original"
 
 
+def test_tensor_valued_keywords_fall_through_without_being_evaluated(plugin, monkeypatch):
+    """An expert map, a bias or zero points arrive as tensors: the dispatch decides on their presence and never
+    asks for their truth value (ambiguous for more than one element, a device sync for one)."""
+    vp, hip_calls = plugin
+    mods, _, calls = _install_fake_vllm(monkeypatch)
+    monkeypatch.setenv(vp.ENV_FLAG, "1")
+    vp.register()
+    fe = mods[vp.FUSED_MOE_MODULE].fused_experts
+    x = _FakeCudaBf16()
+    int8 = dict(use_int8_w8a8=True, per_channel_quant=True, w1_scale=torch.ones(8, 4), w2_scale=torch.ones(8, 4))
+
+    class NoTruth(torch.Tensor):
+        def __bool__(self):
+            raise AssertionError("the dispatch evaluated a tensor")
+
+        def __eq__(self, other):
+            raise AssertionError("the dispatch compared a tensor")
+
+        __hash__ = None
+
+    for other in (dict(expert_map=torch.arange(8)), dict(w1_bias=torch.zeros(8, 4)), dict(w1_zp=torch.zeros(1)),
+                  dict(some_future_tensor=torch.zeros(3)), dict(expert_map=torch.arange(8).as_subclass(NoTruth)),
+                  dict(unknown=torch.zeros(2).as_subclass(NoTruth))):
+        n = len(hip_calls)
+        assert fe(x, 1, 2, 3, 4, **{**int8, **other}) == "original"
+        assert len(hip_calls) == n
+    # tensor-valued scales on the handled path are not evaluated either
+    n = len(hip_calls)
+    scales = dict(w1_scale=torch.ones(8, 4).as_subclass(NoTruth), w2_scale=torch.ones(8, 4).as_subclass(NoTruth))
+    assert fe(x, 1, 2, 3, 4, **{**int8, **scales}, expert_map=None, w1_bias=None) == "hip"
+    assert len(hip_calls) == n + 1
+
+
+def test_rejected_shapes_fall_through_and_runtime_errors_do_not(plugin, monkeypatch):
+    vp, hip_calls = plugin
+    mods, _, calls = _install_fake_vllm(monkeypatch)
+    monkeypatch.setenv(vp.ENV_FLAG, "1")
+    vp.register()
+    fe = mods[vp.FUSED_MOE_MODULE].fused_experts
+    int8 = dict(use_int8_w8a8=True, per_channel_quant=True, w1_scale="s1", w2_scale="s2")
+
+    def meta(*shape, dtype=torch.int8):
+        return torch.empty(shape, dtype=dtype, device="meta")
+
+    class X:
+        is_cuda = True
+        dtype = torch.bfloat16
+        shape = (5, 128)
+
+    ok = (X(), meta(4, 256, 128), meta(4, 128, 128))
+    assert fe(*ok, 3, 4, **int8) == "hip"
+    n = len(hip_calls)
+    # decided from the shapes alone, before the HIP entry is called
+    for w1, w2 in ((meta(4, 256, 96), meta(4, 96, 128)),       # hidden size not a multiple of 64 (and != x)
+                   (meta(4, 200, 128), meta(4, 128, 100)),     # intermediate size not a multiple of 64
+                   (meta(4, 256, 128), meta(4, 128, 64)),      # w2 does not match w1
+                   (meta(2000, 256, 128), meta(2000, 128, 128))):  # more experts than the kernels index
+        assert fe(X(), w1, w2, 3, 4, **int8) == "original"
+    assert fe(*ok, 3, 4, **int8, global_num_experts=16) == "original"  # would need an expert map
+    assert fe(*ok, 3, 4, **{**int8, "w1_scale": None}) == "original"
+    assert len(hip_calls) == n
+    # the entry's own validation may still reject: ValueError falls through like NotImplementedError
+    assert fe(*ok, 3, 4, **{**int8, "w1_scale": "rejected-by-validation"}) == "original"
+    # anything raised while the HIP path runs is a real failure and surfaces
+    with pytest.raises(RuntimeError, match="launch"):
+        fe(*ok, 3, 4, **{**int8, "w1_scale": "launch-failed"})
+
+
 def test_apply_adapter_forwards_to_the_flat_entry(pra, monkeypatch):
     seen = {}
 
@@ -134,6 +207,8 @@ def test_apply_adapter_forwards_to_the_flat_entry(pra, monkeypatch):
 def test_default_workspace_cache_is_bounded(pra, monkeypatch):
     api = pra.api
     monkeypatch.setattr(api, "_workspaces", type(api._workspaces)())
+    monkeypatch.setattr(api, "_pinned_workspaces", set())
+    monkeypatch.setattr(api, "_retired_workspaces", [])
     made = []
     real_empty = torch.empty
 
@@ -151,3 +226,37 @@ def test_default_workspace_cache_is_bounded(pra, monkeypatch):
     n = len(made)
     assert api._workspace(dev, api._MAX_CACHED_WORKSPACES + 4, 512) is made[-1]
     assert len(made) == n
+
+
+def test_pinned_workspaces_are_never_freed(pra, monkeypatch):
+    """A buffer handed out by reserve_workspace or under capture may sit in a captured graph: growing the
+    cache entry retires it to a keep-alive list instead of dropping it, and eviction passes it over."""
+    api = pra.api
+    monkeypatch.setattr(api, "_workspaces", type(api._workspaces)())
+    monkeypatch.setattr(api, "_pinned_workspaces", set())
+    monkeypatch.setattr(api, "_retired_workspaces", [])
+    real_empty = torch.empty
+    monkeypatch.setattr(api.torch, "empty", lambda shape, dtype=None, device=None: real_empty(shape, dtype=dtype))
+    capturing = [False]
+    monkeypatch.setattr(api, "_capturing", lambda device: capturing[0])
+    dev = torch.device("cuda", 0)
+    reserved = api._workspace(dev, 7, 1000, pin=True)
+    assert api._workspace(dev, 7, 800) is reserved
+    grown = api._workspace(dev, 7, 5000)  # eager call above the reserved size
+    assert grown is not reserved and grown.numel() >= 5000
+    assert any(t is reserved for t in api._retired_workspaces)  # still allocated for graphs that hold it
+    # a buffer first used under capture is pinned from then on
+    plain = api._workspace(dev, 8, 1000)
+    capturing[0] = True
+    assert api._workspace(dev, 8, 900) is plain
+    with pytest.raises(RuntimeError, match="reserve_workspace"):
+        api._workspace(dev, 8, 2000)
+    capturing[0] = False
+    bigger = api._workspace(dev, 8, 2000)
+    assert bigger is not plain and any(t is plain for t in api._retired_workspaces)
+    # eviction only ever drops buffers no capture has seen
+    pinned = api._workspace(dev, 9, 64, pin=True)
+    for stream in range(100, 100 + 2 * api._MAX_CACHED_WORKSPACES):
+        api._workspace(dev, stream, 64)
+    assert api._workspaces[(0, 9)] is pinned
+    assert len(api._workspaces) <= api._MAX_CACHED_WORKSPACES
