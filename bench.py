@@ -4,8 +4,9 @@
 A step is one ``fused_experts`` call (quant → align → gate_up GEMM + SiLU·mul → quant → down GEMM →
 combine) on one batch of M tokens of the Qwen3-30B-A3B-shaped layer (E=128, top-8, H=2048, I=768,
 moe_align block 64), inputs resident in HBM.  The headline value is tokens/s at ``--m`` (default
-8192, the prefill point); ``sweep`` repeats the measurement at M = 16, 128, 1024, 8192 and reports
-layer-level INT8 TOP/s and HBM GB/s from the algorithmic work of the sampled routing.  Successive
+8192, the prefill point); ``sweep_detail`` repeats the measurement at M = 16, 128, 512, 1024, 8192 and
+reports layer-level INT8 TOP/s and HBM GB/s from the algorithmic work of the sampled routing; the
+line ends with compact views of the same (``stages``, ``decode_mix``, ``sweep``).  Successive
 steps rotate over several independent weight copies so that no step finds its weights in the
 256 MB last-level cache.
 
@@ -45,8 +46,8 @@ def _profile_traffic(kernel: str, M: int):
     for line in path.read_text().splitlines():
         f = line.split()
         if len(f) == 7 and f[0] == "traffic" and f[1] == kernel and f[2] == f"M={M}":
-            return {"bytes": (float(f[3]) * float(f[5]) + float(f[4]) * float(f[6])) * 1024.0, "source": name}
-    return None
+            return (float(f[3]) * float(f[5]) + float(f[4]) * float(f[6])) * 1024.0, name
+    return None, None
 
 
 def build_workload(pkg, torch, shape_name: str, M: int, copies: int, seed: int):
@@ -486,10 +487,10 @@ def time_other_shape(pkg, torch, oracle, shape_name: str, M: int, steps: int, wa
     P = M * inp.topk_ids.shape[1]
     ids_cpu = inp.topk_ids.cpu()
     ops, nbytes = pkg.inputs.algorithmic_ops(shape, M), pkg.inputs.algorithmic_bytes(shape, M, ids_cpu)
-    line = {"shape": shape_name, "M": M, "routing": shape.routing + (" + shared expert" if shape.shared_expert else ""),
-            "us": t * 1e6, "call_us_p50": ts[len(ts) // 2], "tokens_per_s": M / t,
-            "n_active_experts": int(torch.unique(ids_cpu).numel()), "padded_rows_over_pairs": int(npp.cpu()) / P,
-            "layer_hbm_frac": nbytes / t / PEAK_HBM_BPS, "layer_mfma_frac": ops / t / PEAK_INT8_OPS,
+    r3 = lambda x: float(f"{x:.4g}")
+    line = {"shape": shape_name, "M": M, "us": r3(t * 1e6), "p50_us": r3(ts[len(ts) // 2]),
+            "n_active": int(torch.unique(ids_cpu).numel()), "padded_over_pairs": r3(int(npp.cpu()) / P),
+            "layer_hbm_frac": r3(nbytes / t / PEAK_HBM_BPS), "layer_mfma_frac": r3(ops / t / PEAK_INT8_OPS),
             "bound": "hbm" if nbytes / PEAK_HBM_BPS >= ops / PEAK_INT8_OPS else "mfma"}
     if cpu:
         # only the experts this batch routes to travel to the host (ids remapped), so the checker does the same
@@ -503,8 +504,9 @@ def time_other_shape(pkg, torch, oracle, shape_name: str, M: int, steps: int, wa
         t0 = time.perf_counter()
         oracle.native_w8a8_moe(*args)
         tc = time.perf_counter() - t0
-        line["cpu"] = {"tokens_per_s": M / tc, "s": tc, "cores": torch.get_num_threads(), "kind": "port",
-                       "sample": "whole batch, one pass, no warm-up"}
+        # the CPU checker on the whole batch, one pass, no warm-up
+        line["cpu_tokens_per_s"] = r3(M / tc)
+        line["cpu_cores"] = torch.get_num_threads()
     del inp
     torch.cuda.empty_cache()
     return line
@@ -580,7 +582,10 @@ def main() -> int:
         roof["frac"] = roof["achieved"] / roof["peak"]
         roof["kernel"] = "gemm gate_up + SiLU*mul"
         roof["kernel_us"] = t_k * 1e6
-        roof["traffic"] = _profile_traffic("gate_up", M)
+        # `traffic` = HBM bytes per launch as the hardware counters saw them, a recorded figure (a counter
+        # cannot be read from inside this process): `traffic_source` names the summary it was read from
+        roof["traffic"], roof["traffic_source"] = _profile_traffic("gate_up", M)
+        roof["algorithmic_bytes"] = k_bytes
         point = {
             "M": M,
             "tokens_per_s": M / t_layer,
@@ -622,14 +627,15 @@ def main() -> int:
             "tokens_per_step": args.m,
             "gemm_variant": args.variant,
         },
-        "roofline": {k: headline["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")},
+        "roofline": {k: headline["roofline"][k]
+                     for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "traffic_source", "algorithmic_bytes")},
         "roofline_kernel": headline["roofline"]["kernel"],
         "roofline_kernel_us": headline["roofline"]["kernel_us"],
         "layer_int8_tops": headline["layer_int8_tops"],
         "layer_mfma_frac": headline["layer_mfma_frac"],
         "layer_hbm_gbps": headline["layer_hbm_gbps"],
         "layer_hbm_frac": headline["layer_hbm_frac"],
-        "sweep": sweep,
+        "sweep_detail": sweep,
     }
     if not args.no_sweep:
         out["router"] = [time_router(pkg, torch, pkg.inputs.SHAPES[args.shape], M, args.steps, args.warmup)
@@ -652,6 +658,25 @@ def main() -> int:
         ]
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(oracle, torch, base_headline, args.cpu_sample)
+    # The last keys of the line are a compact view of both targets (whoever keeps only the end of a long
+    # line still sees every batch size): per launch [name, us, fraction of its roofline, bound]; per batch
+    # size the layer time, the p90 of single calls, the layer's fractions of 8 TB/s and of 5 POP/s, and
+    # the gate_up kernel's duration and fraction of the roofline that bounds it.
+    r3 = lambda x: float(f"{x:.4g}")
+    if "decode_mix" in out:
+        dm = out.pop("decode_mix")
+        out["decode_mix_detail"] = dm
+        out["decode_mix"] = {"us_per_layer_call": r3(dm["eager"]["us_per_layer_call"]),
+                             "tokens_per_s": r3(dm["eager"]["tokens_per_s"]),
+                             "hip_graph_us_per_layer_call": r3(dm["hip_graph"]["us_per_layer_call"]),
+                             "layers": dm["layers"], "steps": dm["steps"]}
+    if "stages" in headline:
+        out["stages"] = [[st["stage"], r3(st["us"]), r3(max(st["hbm_frac"], st["mfma_frac"])), st["bound"]]
+                         for st in headline["stages"]]
+    out["sweep"] = [{"M": pt["M"], "us": r3(pt["ms_per_step"] * 1e3), "p90_us": r3(pt["call_us"]["p90"]),
+                     "layer_hbm_frac": r3(pt["layer_hbm_frac"]), "layer_mfma_frac": r3(pt["layer_mfma_frac"]),
+                     "kernel_us": r3(pt["roofline"]["kernel_us"]), "kernel_frac": r3(pt["roofline"]["frac"]),
+                     "bound": pt["roofline"]["bound"]} for pt in sweep]
     print(json.dumps(out))
     return 0
 

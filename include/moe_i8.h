@@ -210,6 +210,17 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
                          void* workspace, int64_t workspace_bytes, int variant, void* stream);
 
 /*
+ * What moe_i8_fused_experts would launch for a layer shape, decided on the host from the sizes alone (no GPU
+ * call): the GEMM kernel of each projection (MOE_I8_GEMM_STREAM, _NARROW, _TILE_WIDE or _TILE_DEEP) and the
+ * number of kernel launches of one call.  A diagnostic with no counterpart in the reference (upstream picks its
+ * kernel configuration from tuned tables per shape): it lets a test pin which measured kernel each benchmark
+ * point runs on, so that a retune of the hand-over points cannot silently move one.  Any output pointer may be
+ * null.  Returns MOE_I8_EUNSUPPORTED when `variant` demands a family that does not handle the shape.
+ */
+int moe_i8_layer_plan(int64_t m, int top_k, int num_experts, int hidden_size, int inter, int block_size,
+                      int variant, int* gate_up_kernel, int* down_kernel, int* launches);
+
+/*
  * moe_i8_fused_experts for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
  * Same arguments and result as moe_i8_fused_experts without the workspace: the intermediate buffers

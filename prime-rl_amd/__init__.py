@@ -11,6 +11,7 @@ from .api import (  # noqa: F401
     fused_experts,
     fused_moe,
     fused_topk,
+    layer_plan,
     grouped_topk,
     route_topk,
     routed_experts_payload,
@@ -25,6 +26,7 @@ from .api import (  # noqa: F401
     per_token_quant_int8,
     quantize_expert_weights,
     load_quantized_expert_weights,
+    load_weights_kernel_int8,
     reserve_workspace,
     quantize_weights_per_channel,
     sorted_capacity,
@@ -35,11 +37,13 @@ from . import api, build, vllm_plugin  # noqa: F401
 __all__ = [
     "fused_experts",
     "fused_moe",
+    "layer_plan",
     "moe_align_block_size",
     "per_token_quant_int8",
     "quantize_weights_per_channel",
     "quantize_expert_weights",
     "load_quantized_expert_weights",
+    "load_weights_kernel_int8",
     "reserve_workspace",
     "moe_sum",
     "fused_topk",

@@ -62,6 +62,7 @@ SIGNATURES = {
         c_int,
         [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, _P, c_int64, c_int, _P],
     ),
+    "moe_i8_layer_plan": (c_int, [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, _P]),
     "moe_i8_fused_experts_static": (
         c_int,
         [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, _P],

@@ -114,6 +114,23 @@ def workspace_bytes(m: int, top_k: int, num_experts: int, hidden: int, inter: in
     return n
 
 
+_KERNEL_NAMES = {_abi.GEMM_STREAM: "stream", _abi.GEMM_NARROW: "narrow", _abi.GEMM_TILE_WIDE: "tile_wide",
+                 _abi.GEMM_TILE_DEEP: "tile_deep"}
+
+
+def layer_plan(m: int, top_k: int, num_experts: int, hidden: int, inter: int,
+               block_size: int = 64, gemm_variant: str | int = "auto") -> dict:
+    """Which GEMM kernel ``fused_experts`` runs for each projection of a layer of this shape and how many
+    kernel launches one call makes: ``{"gate_up": name, "down": name, "launches": n}``.  Decided on the host
+    from the sizes alone (no GPU needed), by the same code the driver uses."""
+    import ctypes
+
+    gu, dn, n = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    _abi.check(_abi.load().moe_i8_layer_plan(m, top_k, num_experts, hidden, inter, block_size, _variant(gemm_variant),
+                                             ctypes.byref(gu), ctypes.byref(dn), ctypes.byref(n)))
+    return {"gate_up": _KERNEL_NAMES[gu.value], "down": _KERNEL_NAMES[dn.value], "launches": n.value}
+
+
 # --------------------------------------------------------------------------------------------- #
 def moe_align_block_size(
     topk_ids: torch.Tensor,
@@ -273,6 +290,35 @@ def quantize_expert_weights(
 _EXPERT_PARAM_SUFFIXES = ("w13_weight", "w13_weight_scale", "w2_weight", "w2_weight_scale")
 
 
+def _resolve_expert_params(params: dict, prefix: str, E: int, I: int, H: int):
+    """The four int8 parameters of the layer ``prefix`` as ``(names, views, missing, mismatches)``: looked up
+    as ``{prefix}.{name}`` or, as the pinned vLLM nests them, ``{prefix}.routed_experts.{name}``
+    (``src/prime_rl/inference/vllm/worker/weight_transfer.py:76-82``); ``views`` are the parameters' tensors
+    in the shapes the quantiser writes (scales may be kept as ``[E, N]`` or ``[E, N, 1]``)."""
+    want = {"w13_weight": (E, 2 * I, H), "w13_weight_scale": (E, 2 * I), "w2_weight": (E, H, I),
+            "w2_weight_scale": (E, H)}
+    names, views, missing, mismatches = {}, {}, [], []
+    for suffix in _EXPERT_PARAM_SUFFIXES:
+        for name in (f"{prefix}.{suffix}", f"{prefix}.routed_experts.{suffix}"):
+            if name in params:
+                break
+        else:
+            missing.append(f"{prefix}.{suffix}")
+            continue
+        param = params[name]
+        t = param.data if isinstance(param, torch.nn.Parameter) else param
+        shape = tuple(t.shape)
+        if shape == want[suffix]:
+            views[suffix] = t
+        elif suffix.endswith("_scale") and shape == want[suffix] + (1,):
+            views[suffix] = t.view(want[suffix])
+        else:
+            mismatches.append(f"{name}: param={list(shape)} != received={list(want[suffix])}")
+            continue
+        names[suffix] = name
+    return names, views, missing, mismatches
+
+
 @torch.no_grad()
 def load_quantized_expert_weights(
     params: dict,
@@ -296,39 +342,138 @@ def load_quantized_expert_weights(
     tensors the way ``tensor[source_indices]`` does there (``:120-125``).  Scales may be ``[E, N]`` or
     ``[E, N, 1]``.  Returns the names written.
     """
-    found, missing = {}, []
-    for suffix in _EXPERT_PARAM_SUFFIXES:
-        for name in (f"{prefix}.{suffix}", f"{prefix}.routed_experts.{suffix}"):
-            if name in params:
-                found[suffix] = (name, params[name])
-                break
-        else:
-            missing.append(f"{prefix}.{suffix}")
-    if missing:
-        raise ValueError(f"int8 expert weight update: {len(missing)} parameters not found in model: {missing}")
     if source_indices is not None:
         idx = source_indices.to(device=w1.device, dtype=torch.long)
         w1, w3, w2 = w1[idx].contiguous(), w3[idx].contiguous(), w2[idx].contiguous()
     if w1.dim() != 3 or w1.shape != w3.shape or w2.dim() != 3:
         raise ValueError("w1 and w3 must be [E, I, H] and w2 [E, H, I]")
     E, I, H = w1.shape
-    want = {"w13_weight": (E, 2 * I, H), "w13_weight_scale": (E, 2 * I), "w2_weight": (E, H, I),
-            "w2_weight_scale": (E, H)}
-    mismatches, views = [], {}
-    for suffix, (name, param) in found.items():
-        t = param.data if isinstance(param, torch.nn.Parameter) else param
-        shape = tuple(t.shape)
-        ok = shape == want[suffix] or (suffix.endswith("_scale") and shape == want[suffix] + (1,))
-        if tuple(w2.shape) != (E, H, I) or not ok:
-            mismatches.append(f"{name}: param={list(shape)} != received={list(want[suffix])}")
-            continue
-        views[suffix] = t.view(want[suffix]) if shape != want[suffix] else t
+    names, views, missing, mismatches = _resolve_expert_params(params, prefix, E, I, H)
+    if missing:
+        raise ValueError(f"int8 expert weight update: {len(missing)} parameters not found in model: {missing}")
+    if tuple(w2.shape) != (E, H, I):
+        mismatches.append(f"{names.get('w2_weight', prefix + '.w2_weight')}: param={[E, H, I]} != received={list(w2.shape)}")
     if mismatches:
         raise ValueError(f"int8 expert weight update had {len(mismatches)} shape mismatches: {mismatches}")
     quantize_expert_weights(
         w1, w3, w2, out=(views["w13_weight"], views["w13_weight_scale"], views["w2_weight"], views["w2_weight_scale"])
     )
-    return [found[suffix][0] for suffix in _EXPERT_PARAM_SUFFIXES]
+    return [names[suffix] for suffix in _EXPERT_PARAM_SUFFIXES]
+
+
+# incoming names of routed-expert weights -> (role, layer prefix).  Trainer format
+# (``src/prime_rl/trainer/models/glm_moe_dsa/converting_glm_moe_dsa.py:97-99``): ``...experts.gate_proj``,
+# ``...experts.up_proj``, ``...experts.down_proj``; kernel format with bf16 payload (``:123-125``):
+# ``...experts.w13_weight`` (gate rows, then up rows) and ``...experts.w2_weight``.
+_EXPERT_ROLE_SUFFIXES = (
+    (".experts.gate_proj", "w1"), (".experts.up_proj", "w3"), (".experts.down_proj", "w2"),
+    (".experts.routed_experts.w13_weight", "w13"), (".experts.routed_experts.w2_weight", "w2"),
+    (".experts.w13_weight", "w13"), (".experts.w2_weight", "w2"),
+)
+
+
+def _expert_role(name: str):
+    for suffix, role in _EXPERT_ROLE_SUFFIXES:
+        if name.endswith(suffix):
+            return role, name[: len(name) - len(suffix)] + ".experts"
+    return None, None
+
+
+@torch.no_grad()
+def load_weights_kernel_int8(model, state_iter, expert_source_indices: dict | None = None) -> dict:
+    """Policy update of a whole int8 W8A8 model from the trainer's ``(name, tensor)`` stream: the int8
+    counterpart of the reference's ``load_weights_kernel``
+    (``src/prime_rl/inference/vllm/worker/weight_transfer.py:97-134``).
+
+    ``model`` is the engine's module (its ``named_parameters()`` are used) or such a dict.  bf16
+    routed-expert weights are collected per layer — ``w1``/``w3``/``w2`` under the trainer's names, or
+    ``w13_weight``/``w2_weight`` in kernel format — and, once a layer is complete, quantised per output
+    channel and written in place into that layer's ``w13_weight``, ``w13_weight_scale``, ``w2_weight``,
+    ``w2_weight_scale`` (flat or nested under ``routed_experts``).  Every other tensor is copied in place
+    into the parameter of the same name (tried flat, then with the ``routed_experts`` nesting), exactly as
+    the reference does; that includes weights that arrive already quantised.  ``expert_source_indices``
+    maps a module-name prefix to the experts local to this worker (``weight_transfer.py:76-95,120-125``).
+
+    Nothing raises midway: names that are not in the model, tensors whose shapes do not match and expert
+    groups that never became complete are collected, everything else is written, and ONE ``ValueError``
+    at the end lists them all (mismatches first, as the reference orders its two errors).  Returns
+    ``{"loaded": [...names written...], "quantized_layers": [...prefixes...]}``.
+    """
+    params = dict(model.named_parameters()) if hasattr(model, "named_parameters") else dict(model)
+    expert_source_indices = expert_source_indices or {}
+    loaded, layers, skipped, mismatches = [], [], [], []
+    pending: dict[str, dict[str, tuple[str, torch.Tensor]]] = {}
+
+    def local_experts(prefix: str, t: torch.Tensor) -> torch.Tensor:
+        for module_name, idx in expert_source_indices.items():
+            if prefix.startswith(f"{module_name}.") or prefix == module_name:
+                return t[idx.to(device=t.device, dtype=torch.long)].contiguous()
+        return t
+
+    def flush(prefix: str, group: dict) -> None:
+        w2 = local_experts(prefix, group["w2"][1])
+        if "w13" in group:
+            w13 = local_experts(prefix, group["w13"][1])
+            if w13.dim() != 3 or w13.shape[1] % 2 or w2.dim() != 3:
+                mismatches.append(f"{group['w13'][0]}: received={list(w13.shape)} is not [E, 2I, H]")
+                return
+            E, I, H = w13.shape[0], w13.shape[1] // 2, w13.shape[2]
+        else:
+            w1, w3 = local_experts(prefix, group["w1"][1]), local_experts(prefix, group["w3"][1])
+            if w1.dim() != 3 or w1.shape != w3.shape or w2.dim() != 3:
+                mismatches.append(f"{group['w1'][0]}: received={list(w1.shape)} / {list(w3.shape)} are not two [E, I, H]")
+                return
+            E, I, H = w1.shape
+        names, views, missing, bad = _resolve_expert_params(params, prefix, E, I, H)
+        if tuple(w2.shape) != (E, H, I):
+            bad.append(f"{group['w2'][0]}: param={[E, H, I]} != received={list(w2.shape)}")
+        if missing or bad:
+            skipped.extend(missing)
+            mismatches.extend(bad)
+            return
+        out = (views["w13_weight"], views["w13_weight_scale"], views["w2_weight"], views["w2_weight_scale"])
+        if "w13" in group:
+            quantize_weights_per_channel(w13.contiguous(), out=out[:2])
+            quantize_weights_per_channel(w2.contiguous(), out=out[2:])
+        else:
+            quantize_expert_weights(w1.contiguous(), w3.contiguous(), w2.contiguous(), out=out)
+        loaded.extend(names[suffix] for suffix in _EXPERT_PARAM_SUFFIXES)
+        layers.append(prefix)
+
+    for name, tensor in state_iter:
+        role, prefix = _expert_role(name)
+        if role is not None and tensor.dtype == torch.bfloat16:
+            group = pending.setdefault(prefix, {})
+            group[role] = (name, tensor)
+            if "w2" in group and ("w13" in group or ("w1" in group and "w3" in group)):
+                flush(prefix, pending.pop(prefix))
+            continue
+        target = name
+        if target not in params and ".experts." in name and ".routed_experts." not in name:
+            head, _, tail = name.rpartition(".experts.")
+            target = f"{head}.experts.routed_experts.{tail}"
+        if target not in params:
+            skipped.append(name)
+            continue
+        param = params[target]
+        if tuple(param.shape) != tuple(tensor.shape):
+            prefix_of = target.rpartition(".")[0]
+            tensor = local_experts(prefix_of, tensor) if expert_source_indices else tensor
+            if tuple(param.shape) != tuple(tensor.shape):
+                mismatches.append(f"{target}: param={list(param.shape)} != received={list(tensor.shape)}")
+                continue
+        param.copy_(tensor)
+        loaded.append(target)
+    for prefix, group in pending.items():
+        skipped.extend(f"{n} (incomplete expert group of {prefix}: got {sorted(group)})" for n, _ in group.values())
+    if mismatches or skipped:
+        parts = []
+        if mismatches:
+            parts.append(f"{len(mismatches)} shape mismatches: {mismatches}")
+        if skipped:
+            parts.append(f"skipped {len(skipped)} weights not found in model: {skipped}")
+        raise ValueError("int8 kernel weight transfer had " + "; ".join(parts))
+    return {"loaded": loaded, "quantized_layers": layers}
 
 
 def moe_sum(input: torch.Tensor, output: torch.Tensor) -> None:

@@ -463,6 +463,11 @@ int64_t align_workspace_ints(int64_t num_pairs, int num_experts) {
   return 2 * units * num_experts + num_experts + 1;
 }
 
+// Launches launch_align (and launch_align_quant) make for this many pairs.
+int align_launches(const AlignArgs& a) {
+  return a.num_pairs <= kSingleMaxPairs ? 1 : a.num_pairs <= kChunkedMaxPairs ? 2 : 3;
+}
+
 bool align_quant_fusable(const AlignArgs& a, const QuantArgs& q) {
   if (q.rows <= 0 || q.rows > (int64_t)kSingleWaves * 0x7ffffff0) return false;
   return a.num_pairs > kSingleMaxPairs || q.rows <= kSingleMaxPairs;

@@ -112,6 +112,42 @@ int run_gemm(const moe_i8::GemmArgs& g0, int variant, hipStream_t stream) {
   }
 }
 
+moe_i8::GemmArgs gate_up_args(const int8_t* x_q, const float* a_scale, const int8_t* w1, const float* w1_scale,
+                              const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                              const int32_t* num_tokens_post_padded, int64_t num_pairs, int top_k, int num_experts,
+                              int hidden, int inter, int block_size, int64_t sorted_cap, void* act_out) {
+  moe_i8::GemmArgs g{};
+  g.mode = moe_i8::kGateUpSilu;
+  g.a_q = x_q;
+  g.a_scale = a_scale;
+  g.w = w1;
+  g.w_scale = w1_scale;
+  g.row_weight = nullptr;
+  g.sorted_token_ids = sorted_token_ids;
+  g.expert_ids = expert_ids;
+  g.num_tokens_post_padded = num_tokens_post_padded;
+  g.num_pairs = num_pairs;
+  g.row_div = top_k;
+  g.num_experts = num_experts;
+  g.n = 2 * inter;
+  g.k = hidden;
+  g.block_size = block_size;
+  g.sorted_cap = sorted_cap;
+  g.out = act_out;
+  g.max_rows_per_expert = (num_pairs + top_k - 1) / top_k;  // an expert sees a token at most once
+  return g;
+}
+
+// The family of `picks_family` with the geometry of the LDS-tiled family spelled out
+// (MOE_I8_GEMM_STREAM, _NARROW, _TILE_WIDE or _TILE_DEEP); -1 as there.
+int picks_kernel(const moe_i8::GemmArgs& g0, int variant) {
+  const int family = picks_family(g0, variant);
+  if (family != MOE_I8_GEMM_TILE) return family;
+  moe_i8::GemmArgs g = g0;
+  g.tile_geometry = tile_geometry_of(variant);
+  return moe_i8::gemm_tile_geometry(g) == moe_i8::kTileDeep ? MOE_I8_GEMM_TILE_DEEP : MOE_I8_GEMM_TILE_WIDE;
+}
+
 moe_i8::GemmArgs down_args(const int8_t* h_q, const float* a_scale, const int8_t* w2, const float* w2_scale,
                            const float* topk_weights, const int32_t* sorted_token_ids, const int32_t* expert_ids,
                            const int32_t* num_tokens_post_padded, int64_t num_pairs, int num_experts, int hidden,
@@ -332,25 +368,8 @@ static int gemm_gate_up_impl(const int8_t* x_q, const float* a_scale, const int8
   if (!a_scale || !w1_scale) return fail(MOE_I8_EINVAL, "null scale pointer");
   if (!aligned16(w1_scale)) return fail(MOE_I8_EINVAL, "w1_scale must be 16-byte aligned");
   if (top_k < 1) return fail(MOE_I8_EINVAL, "top_k must be >= 1");
-  moe_i8::GemmArgs g{};
-  g.mode = moe_i8::kGateUpSilu;
-  g.a_q = x_q;
-  g.a_scale = a_scale;
-  g.w = w1;
-  g.w_scale = w1_scale;
-  g.row_weight = nullptr;
-  g.sorted_token_ids = sorted_token_ids;
-  g.expert_ids = expert_ids;
-  g.num_tokens_post_padded = num_tokens_post_padded;
-  g.num_pairs = num_pairs;
-  g.row_div = top_k;
-  g.num_experts = num_experts;
-  g.n = 2 * inter;
-  g.k = hidden;
-  g.block_size = block_size;
-  g.sorted_cap = sorted_cap;
-  g.out = act_out;
-  g.max_rows_per_expert = (num_pairs + top_k - 1) / top_k;  // an expert sees a token at most once
+  moe_i8::GemmArgs g = gate_up_args(x_q, a_scale, w1, w1_scale, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                                    num_pairs, top_k, num_experts, hidden, inter, block_size, sorted_cap, act_out);
   g.expert_ids_ascend = from_align;
   return run_gemm(g, variant, static_cast<hipStream_t>(stream));
 }
@@ -491,6 +510,50 @@ Carve carve(int64_t m, int top_k, int num_experts, int hidden, int inter, int bl
   c.total = off;
   return c;
 }
+
+// What moe_i8_fused_experts launches for a layer shape: decided on the host from the sizes alone.
+struct LayerPlan {
+  int gate_up_kernel;   // MOE_I8_GEMM_STREAM, _NARROW, _TILE_WIDE or _TILE_DEEP; -1 = shape not supported by the demanded family
+  int down_kernel;
+  bool fuse_align_quant;  // moe_align and the quantisation of the layer input in one launch
+  bool down_quantises;    // the streaming down GEMM quantises its own bf16 activations (one launch less)
+  int launches;
+};
+
+LayerPlan plan_layer(int64_t m, int top_k, int num_experts, int hidden, int inter, int block_size, int variant) {
+  const Carve c = carve(m, top_k, num_experts, hidden, inter, block_size);
+  const int64_t p = m * top_k;
+  LayerPlan plan{};
+  moe_i8::GemmArgs gu = gate_up_args(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, p, top_k, num_experts,
+                                     hidden, inter, block_size, c.cap, nullptr);
+  gu.expert_ids_ascend = true;
+  plan.gate_up_kernel = picks_kernel(gu, variant);
+  moe_i8::GemmArgs dg = down_args(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, p, num_experts,
+                                  hidden, inter, block_size, c.cap, nullptr);
+  dg.expert_ids_ascend = true;
+  dg.max_rows_per_expert = m;
+  plan.down_kernel = picks_kernel(dg, variant);
+  // Very few rows per expert (decode): the streaming down GEMM quantises its activations itself, one
+  // launch less.  Every workgroup of a block repeats that quantisation, so from about four rows
+  // per expert on (measured) the separate launch is the cheaper one again.
+  plan.down_quantises = plan.down_kernel == MOE_I8_GEMM_STREAM && moe_i8::gemm_stream_fuses_quant(inter) &&
+                        p <= (int64_t)3 * num_experts;
+  moe_i8::AlignArgs aa{};
+  aa.num_pairs = p;
+  aa.num_experts = num_experts;
+  aa.block_size = block_size;
+  aa.sorted_cap = c.cap;
+  aa.expert_cap = c.ecap;
+  moe_i8::QuantArgs qa{};
+  qa.src_rows = m;
+  qa.cols = hidden;
+  qa.row_stride = hidden;
+  qa.gather_div = 1;
+  qa.rows = m;
+  plan.fuse_align_quant = moe_i8::align_quant_fusable(aa, qa);
+  plan.launches = moe_i8::align_launches(aa) + (plan.fuse_align_quant ? 0 : 1) + 1 + (plan.down_quantises ? 1 : 2) + 1;
+  return plan;
+}
 }  // namespace
 
 int64_t moe_i8_workspace_bytes(int64_t m, int top_k, int num_experts, int hidden, int inter,
@@ -528,6 +591,9 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
   float* a2 = reinterpret_cast<float*>(ws + c.a2);
   void* down = ws + c.down;
   const int64_t p = m * top_k;
+
+  const LayerPlan plan = plan_layer(m, top_k, num_experts, hidden_size, inter, block_size, variant);
+  if (plan.gate_up_kernel < 0 || plan.down_kernel < 0) return MOE_I8_EUNSUPPORTED;
 
   // Small batches: moe_align (one workgroup) and the quantisation of the input share one launch.
   moe_i8::AlignArgs aa;
@@ -567,15 +633,7 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
   if (int rc = gemm_gate_up_impl(x_q, a1, w1, w1_scale, sorted, eids, npp, p, top_k, num_experts, hidden_size, inter,
                                  block_size, c.cap, act, variant, true, stream))
     return rc;
-  // Very few rows per expert (decode): the streaming down GEMM quantises its activations itself, one
-  // launch less.  Every workgroup of a block repeats that quantisation, so from about four rows
-  // per expert on (measured) the separate launch is the cheaper one again.
-  moe_i8::GemmArgs dg = down_args(act_q, a2, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
-                                  hidden_size, inter, block_size, c.cap, down);
-  dg.expert_ids_ascend = true;
-  const int down_family = picks_family(dg, variant);
-  if (down_family < 0) return MOE_I8_EUNSUPPORTED;
-  if (down_family == MOE_I8_GEMM_STREAM && moe_i8::gemm_stream_fuses_quant(inter) && p <= (int64_t)3 * num_experts) {
+  if (plan.down_quantises) {
     if (int rc = moe_i8_gemm_down_bf16(act, w2, w2_scale, topk_weights, sorted, eids, npp, p, num_experts,
                                        hidden_size, inter, block_size, c.cap, down, stream))
       return rc;
@@ -587,6 +645,24 @@ int moe_i8_fused_experts(const void* hidden, const int8_t* w1, const int8_t* w2,
       return rc;
   }
   return moe_i8_sum(down, out, m, top_k, hidden_size, stream);
+}
+
+int moe_i8_layer_plan(int64_t m, int top_k, int num_experts, int hidden_size, int inter, int block_size,
+                      int variant, int* gate_up_kernel, int* down_kernel, int* launches) {
+  if (m < 1 || top_k < 1 || m * top_k > INT32_MAX - 1) return fail(MOE_I8_EINVAL, "m / top_k out of range");
+  if (num_experts < 1 || num_experts > MOE_I8_MAX_EXPERTS)
+    return fail(MOE_I8_EINVAL, "num_experts must be in [1, %d]", MOE_I8_MAX_EXPERTS);
+  if (!valid_block_size(block_size)) return fail(MOE_I8_EINVAL, "block_size must be 16, 32, 64 or 128");
+  if (hidden_size < 64 || hidden_size % 64 || inter < 64 || inter % 64)
+    return fail(MOE_I8_EINVAL, "hidden (%d) and inter (%d) must be positive multiples of 64", hidden_size, inter);
+  if (variant < MOE_I8_GEMM_AUTO || variant > MOE_I8_GEMM_TILE_DEEP)
+    return fail(MOE_I8_EINVAL, "unknown GEMM variant %d", variant);
+  const LayerPlan plan = plan_layer(m, top_k, num_experts, hidden_size, inter, block_size, variant);
+  if (plan.gate_up_kernel < 0 || plan.down_kernel < 0) return MOE_I8_EUNSUPPORTED;
+  if (gate_up_kernel) *gate_up_kernel = plan.gate_up_kernel;
+  if (down_kernel) *down_kernel = plan.down_kernel;
+  if (launches) *launches = plan.launches;
+  return MOE_I8_OK;
 }
 
 // ---- the entry point that allocates nothing ----

@@ -138,6 +138,7 @@ struct AlignArgs {
 };
 int64_t align_workspace_ints(int64_t num_pairs, int num_experts);
 hipError_t launch_align(const AlignArgs& a, hipStream_t stream);
+int align_launches(const AlignArgs& a);  // 1, 2 or 3 by the number of pairs
 
 struct QuantArgs {
   const uint16_t* x;  // bf16 bits
@@ -233,6 +234,7 @@ bool gemm_stream_fuses_quant(int k);  // the down GEMM can quantise bf16 activat
 hipError_t launch_gemm_tile(const GemmArgs& a, hipStream_t stream);
 bool gemm_tile_supports(const GemmArgs& a);
 bool gemm_tile_prefers_deep(const GemmArgs& a);
+int gemm_tile_geometry(const GemmArgs& a);  // kTileWide or kTileDeep: what a launch of the family would use
 hipError_t launch_gemm_narrow(const GemmArgs& a, hipStream_t stream);
 bool gemm_narrow_supports(const GemmArgs& a);
 

@@ -746,15 +746,15 @@ bool gemm_tile_prefers_deep(const GemmArgs& a) {
   return a.num_pairs <= (int64_t)kTileDeepRowsPerExpert * a.num_experts;
 }
 
+// The geometry a launch of this family uses for `a` (kTileWide or kTileDeep).
+int gemm_tile_geometry(const GemmArgs& a) {
+  if (a.tile_geometry == kTileWide) return kTileWide;
+  if (a.tile_geometry == kTileDeep) return kTileDeep;
+  return geometry_supports<true>(a) && (gemm_tile_prefers_deep(a) || !geometry_supports<false>(a)) ? kTileDeep : kTileWide;
+}
+
 hipError_t launch_gemm_tile(const GemmArgs& a, hipStream_t stream) {
-  bool deep;
-  if (a.tile_geometry == kTileWide)
-    deep = false;
-  else if (a.tile_geometry == kTileDeep)
-    deep = true;
-  else
-    deep = geometry_supports<true>(a) && (gemm_tile_prefers_deep(a) || !geometry_supports<false>(a));
-  if (deep) {
+  if (gemm_tile_geometry(a) == kTileDeep) {
     switch (a.mode) {
       case kGateUpSilu: return launch_mode<kGateUpSilu, true>(a, stream);
       case kDown: return launch_mode<kDown, true>(a, stream);

@@ -20,7 +20,9 @@ Two surfaces are covered:
   returning a ``MoERunner``, reference ``src/prime_rl/inference/vllm/worker/weight_transfer.py:76-82``;
   the choice of experts implementation goes through ``FusedMoEConfig``, ``patches.py:740-757``):
   ``Int8W8A8HipExperts`` has the ``apply(output, hidden_states, w1, w2, topk_weights, topk_ids, ...)``
-  shape of an experts implementation and forwards to the same C-ABI driver.
+  shape of an experts implementation and forwards to the same C-ABI driver;
+  ``register_experts_selection()`` makes the int8 W8A8 quantisation method's ``select_gemm_impl`` return
+  it for layers this library can take.
 
 Nothing here allocates under HIP graph capture: a call made while the stream is capturing uses a
 workspace that was allocated beforehand for that (device, stream) by ``reserve_workspace`` or by an
@@ -125,10 +127,7 @@ def _wrap(original, hip_fused_experts=None):
     return fused_experts
 
 
-def register() -> bool:
-    """Entry point for ``vllm.general_plugins``. Returns True when a patch was applied."""
-    if os.environ.get(ENV_FLAG, "0") != "1":
-        return False
+def _register_flat() -> bool:
     try:
         fm = importlib.import_module(FUSED_MOE_MODULE)
     except ImportError:
@@ -144,6 +143,87 @@ def register() -> bool:
         if getattr(mod, "fused_experts", None) is original:
             mod.fused_experts = patched
     return True
+
+
+# Where the engine picks the experts implementation of an int8 W8A8 MoE layer: the quantisation method's
+# ``select_gemm_impl(prepare_finalize, layer)`` returns the object whose ``apply`` the modular kernel calls.
+# (Class and module names as vLLM publishes them for channel-wise int8 compressed-tensors checkpoints; override
+# with PRIME_MOE_I8_HIP_METHOD="module:Class[,module:Class...]" for another quantisation method.)
+MODULAR_METHODS = (
+    ("vllm.model_executor.layers.quantization.compressed_tensors.compressed_tensors_moe",
+     "CompressedTensorsW8A8Int8MoEMethod"),
+)
+ENV_METHODS = "PRIME_MOE_I8_HIP_METHOD"
+
+
+def _layer_eligible(method, layer) -> bool:
+    """Channel-wise int8 weights with dynamic per-token activation scales, SiLU, every expert local."""
+    w13, w2 = getattr(layer, "w13_weight", None), getattr(layer, "w2_weight", None)
+    s13, s2 = getattr(layer, "w13_weight_scale", None), getattr(layer, "w2_weight_scale", None)
+    if w13 is None or w2 is None or s13 is None or s2 is None:
+        return False
+    if str(getattr(w13, "dtype", "")) != "torch.int8" or str(getattr(w2, "dtype", "")) != "torch.int8":
+        return False
+    if getattr(layer, "expert_map", None) is not None or getattr(layer, "_expert_map", None) is not None:
+        return False
+    if getattr(layer, "activation", "silu") != "silu":
+        return False
+    if getattr(method, "static_input_scales", False) is True:
+        return False
+    if getattr(layer, "w13_input_scale", None) is not None or getattr(layer, "w2_input_scale", None) is not None:
+        return False
+    probe = type("x", (), {"shape": (1, w13.shape[-1])})()
+    return _shapes_eligible(probe, w13, w2, {})
+
+
+def _wrap_select_gemm_impl(original):
+    def select_gemm_impl(self, prepare_finalize, layer, *args, **kwargs):
+        if _layer_eligible(self, layer):
+            return Int8W8A8HipExperts(layer.w13_weight_scale, layer.w2_weight_scale)
+        return original(self, prepare_finalize, layer, *args, **kwargs)
+
+    setattr(select_gemm_impl, _MARK, True)
+    select_gemm_impl.__wrapped__ = original
+    return select_gemm_impl
+
+
+def register_experts_selection() -> bool:
+    """Put ``Int8W8A8HipExperts`` where the engine selects a MoE layer's experts implementation, the way the
+    reference steers that selection by patching a class of the pinned vLLM in every process
+    (``src/prime_rl/inference/patches.py:740-757``, gated by an environment variable as in
+    ``src/prime_rl/inference/vllm/worker/__init__.py:12-22``): ``select_gemm_impl`` of the int8 W8A8 MoE
+    quantisation method returns the HIP experts for layers this library can take and defers to the original
+    otherwise.  Idempotent; returns True when at least one class was patched.  Exercised on the CPU against a
+    stand-in class; which class the pinned vLLM uses can only be confirmed on a machine that has it, hence the
+    override variable."""
+    if os.environ.get(ENV_FLAG, "0") != "1":
+        return False
+    targets = list(MODULAR_METHODS)
+    override = os.environ.get(ENV_METHODS, "")
+    if override:
+        targets = [tuple(item.split(":", 1)) for item in override.split(",") if ":" in item]
+    patched_any = False
+    for module_name, class_name in targets:
+        try:
+            cls = getattr(importlib.import_module(module_name), class_name, None)
+        except ImportError:
+            continue
+        original = getattr(cls, "select_gemm_impl", None) if cls is not None else None
+        if original is None or getattr(original, _MARK, False):
+            continue
+        cls.select_gemm_impl = _wrap_select_gemm_impl(original)
+        patched_any = True
+    return patched_any
+
+
+def register() -> bool:
+    """Entry point for ``vllm.general_plugins``. Returns True when a patch was applied: the flat
+    ``fused_experts`` function is rebound and the experts selection of the modular-kernel path is steered."""
+    if os.environ.get(ENV_FLAG, "0") != "1":
+        return False
+    flat = _register_flat()
+    modular = register_experts_selection()
+    return flat or modular
 
 
 def reserve_workspace(max_tokens: int, top_k: int, num_experts: int, hidden: int, inter: int, device=None,

@@ -212,3 +212,50 @@ def test_header_is_plain_c_and_a_c_client_links(pra, tmp_path):
     subprocess.run(cmd, check=True, capture_output=True, text=True)
     run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
     assert run.returncode == 0 and run.stdout.strip() == "ok", run.stdout + run.stderr
+
+
+# Which kernel the library picks by itself at every benchmark point (shape, tokens) and how many launches a
+# layer call makes there.  These are the kernels the committed measurements were taken on: a retune of the
+# hand-over points between the GEMM families must change this table knowingly.
+_PLAN = [
+    ("toy", 256, "tile_deep", "tile_deep", 5),
+    ("qwen3-30b-a3b", 1, "stream", "stream", 4),
+    ("qwen3-30b-a3b", 16, "stream", "stream", 4),
+    ("qwen3-30b-a3b", 128, "stream", "stream", 5),
+    ("qwen3-30b-a3b", 256, "narrow", "narrow", 5),
+    ("qwen3-30b-a3b", 512, "narrow", "narrow", 5),
+    ("qwen3-30b-a3b", 1024, "tile_deep", "tile_deep", 5),
+    ("qwen3-30b-a3b", 8192, "tile_wide", "tile_wide", 7),
+    ("glm-4.5-air", 32, "stream", "stream", 5),
+    ("glm-4.5-air", 512, "tile_deep", "tile_deep", 5),
+    ("glm-4.5-air", 4096, "tile_wide", "tile_wide", 7),
+    ("deepseek-v3", 8, "stream", "stream", 5),
+    ("deepseek-v3", 64, "stream", "stream", 5),
+    ("deepseek-v3", 2048, "tile_deep", "tile_deep", 6),
+    ("deepseek-v3", 16384, "tile_wide", "tile_wide", 7),
+]
+
+
+@pytest.mark.parametrize("shape_name,M,gate_up,down,launches", _PLAN)
+def test_kernel_choice_at_the_benchmark_points(pra, shape_name, M, gate_up, down, launches):
+    shape = pra.inputs.SHAPES[shape_name]
+    k = shape.k + (1 if shape.shared_expert else 0)
+    plan = pra.layer_plan(M, k, shape.E_total, shape.H, shape.I)
+    assert plan == {"gate_up": gate_up, "down": down, "launches": launches}
+
+
+def test_layer_plan_follows_a_demanded_family_and_rejects_what_it_cannot_run(pra):
+    abi = pra._abi
+    assert pra.layer_plan(8192, 8, 128, 2048, 768, gemm_variant="stream") == {
+        "gate_up": "stream", "down": "stream", "launches": 7}
+    assert pra.layer_plan(1024, 8, 128, 2048, 768, gemm_variant="tile_wide")["gate_up"] == "tile_wide"
+    assert pra.layer_plan(1024, 8, 128, 2048, 768, gemm_variant="tile")["gate_up"] == "tile_deep"
+    with pytest.raises(abi.MoeI8Error) as e:  # the tiled families take blocks of 64 or 128 rows only
+        pra.layer_plan(1024, 8, 128, 2048, 768, block_size=16, gemm_variant="tile_wide")
+    assert e.value.code == abi.EUNSUPPORTED
+    with pytest.raises(abi.MoeI8Error):
+        pra.layer_plan(0, 8, 128, 2048, 768)
+    with pytest.raises(abi.MoeI8Error):
+        pra.layer_plan(16, 8, 128, 2048, 700)
+    # output pointers are optional
+    assert abi.load().moe_i8_layer_plan(16, 8, 128, 2048, 768, 64, abi.GEMM_AUTO, None, None, None) == abi.OK

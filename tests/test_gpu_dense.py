@@ -99,3 +99,26 @@ def test_gated_mlp_of_a_few_rows_equals_the_rows_of_a_larger_call(pra, H, I, m):
     big = pra.w8a8_mlp(x, *args)
     small = pra.w8a8_mlp(x[:m].contiguous(), *args)
     assert torch.equal(small, big[:m]), int((small != big[:m]).sum())
+
+
+def test_caller_owned_workspace_for_the_dense_ops(pra):
+    """``workspace=`` of ``apply_int8_linear`` and ``w8a8_mlp``: the caller's buffer is used (bit-equal to the
+    default call, also when the buffer starts out as garbage) and one that is too small is refused."""
+    g = torch.Generator().manual_seed(11)
+    M, H, I = 70, 512, 256
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16).to(DEV)
+    w13, s13 = _weights(2 * I, H, g)
+    w2, s2 = _weights(H, I, g)
+    args = (w13.to(DEV), (s13 * 0.3).to(DEV), w2.to(DEV), (s2 * 0.3).to(DEV))
+    lib = pra._abi.load()
+    need = max(lib.moe_i8_dense_workspace_bytes(M, H, I), lib.moe_i8_dense_workspace_bytes(M, H, 0))
+    ws = torch.full((need,), 0xA5, dtype=torch.uint8, device=DEV)
+    want = pra.w8a8_mlp(x, *args)
+    assert torch.equal(pra.w8a8_mlp(x, *args, workspace=ws), want)
+    lin = pra.apply_int8_linear(x, args[0], args[1])
+    ws.fill_(0x3C)
+    assert torch.equal(pra.apply_int8_linear(x, args[0], args[1], workspace=ws), lin)
+    with pytest.raises(ValueError):
+        pra.w8a8_mlp(x, *args, workspace=ws[:64])
+    with pytest.raises(ValueError):
+        pra.apply_int8_linear(x, args[0], args[1], workspace=ws[:64])

@@ -140,6 +140,20 @@ def test_hip_graph_replay(pra, M):
         torch.cuda.synchronize()
         assert torch.equal(out, eager), i
         assert torch.equal(_run(pra, inp), eager)
+    # another batch copied into the captured input tensors: the replay must follow it (kernels that ran
+    # eagerly during the capture instead of being recorded would leave the old result in place)
+    other = im.make_inputs("qwen3-30b-a3b", M, seed=44).to(DEV)
+    static_x.copy_(other.hidden_states)
+    inp.topk_weights.copy_(other.topk_weights)
+    inp.topk_ids.copy_(other.topk_ids)
+    want = pra.fused_experts(other.hidden_states, inp.w1, inp.w2, other.topk_weights, other.topk_ids,
+                             **inp.fused_experts_kwargs())
+    assert not torch.equal(want, eager)
+    out.zero_()
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
 
 
 def test_decode_mix_sequence_reuses_workspace(pra, oracle):
@@ -262,6 +276,88 @@ def test_capture_never_allocates_the_default_workspace(pra):
             # eager work at the reserved size on the same stream between replays: same buffer, no regrowth
             pra.fused_experts(*big.fused_experts_args(), **big.fused_experts_kwargs())
             torch.cuda.synchronize()
+
+
+def test_captured_graph_survives_a_larger_eager_call(pra):
+    """A graph captured against the default workspace keeps replaying correctly after an eager call on the
+    same stream has needed a larger one: the buffer the graph holds stays allocated (it is retired, not
+    freed) and is not handed to anything else."""
+    im = inputs_mod()
+    api = pra.api
+    shape = im.SHAPES["qwen3-30b-a3b"]
+    inp = im.make_inputs(shape, 32, seed=15).to(DEV)
+    big = im.make_inputs(shape, 256, seed=16).to(DEV)
+    eager = _run(pra, inp)
+    eager_big = _run(pra, big)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        reserved = pra.reserve_workspace(32, shape.k, shape.E_total, shape.H, shape.I)
+        key = (reserved.device.index, stream.cuda_stream)
+        assert api._workspaces[key] is reserved
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            out = pra.fused_experts(*inp.fused_experts_args(), **inp.fused_experts_kwargs())
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        # larger than reserved, same stream, eager: the cache entry grows by replacement ...
+        got_big = pra.fused_experts(*big.fused_experts_args(), **big.fused_experts_kwargs())
+        torch.cuda.synchronize()
+        assert torch.equal(got_big, eager_big)
+        grown = api._workspaces[key]
+        assert grown is not reserved and grown.numel() > reserved.numel()
+        # ... and the captured buffer is still referenced, so the allocator cannot hand it out again
+        assert any(t is reserved for t in api._retired_workspaces)
+        fill = [torch.full((reserved.numel(),), 0x5A, dtype=torch.uint8, device=DEV) for _ in range(4)]
+        assert all(f.data_ptr() != reserved.data_ptr() for f in fill)
+        for _ in range(3):
+            out.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager)
+            assert all(bool((f == 0x5A).all()) for f in fill)  # the replay wrote nothing outside its own buffer
+            assert torch.equal(pra.fused_experts(*big.fused_experts_args(), **big.fused_experts_kwargs()), eager_big)
+            torch.cuda.synchronize()
+
+
+def test_apply_adapter_and_out_keyword_on_device(pra, oracle):
+    """The modular-kernel adapter (``Int8W8A8HipExperts.apply(output, hidden_states, w1, w2, topk_weights,
+    topk_ids, ...)``) and the ``out=`` keyword of ``fused_experts`` on device tensors: the caller's tensor is
+    written, bit-equal to the plain call, within tolerance of the oracle; ``out`` may alias the input."""
+    im = inputs_mod()
+    for name, M in (("toy", 100), ("qwen3-30b-a3b", 48)):
+        inp = im.make_inputs(name, M, seed=31).to(DEV)
+        plain = _run(pra, inp)
+        cpu = inp.to("cpu")
+        want = oracle.fused_experts(cpu.hidden_states, cpu.w1, cpu.w2, cpu.topk_weights, cpu.topk_ids,
+                                    cpu.w1_scale, cpu.w2_scale, 64)
+        assert rel_err(plain, want) < TOL
+        # out=
+        out = torch.full_like(inp.hidden_states, float("nan"))
+        ret = pra.fused_experts(*inp.fused_experts_args(), out=out, **inp.fused_experts_kwargs())
+        assert ret is out and torch.equal(out, plain)
+        # the adapter: output first, vLLM's keyword names, its two workspaces ignored
+        experts = pra.vllm_plugin.Int8W8A8HipExperts(inp.w1_scale, inp.w2_scale)
+        output = torch.full_like(inp.hidden_states, float("nan"))
+        before = output.data_ptr()
+        junk = torch.empty(16, device=DEV)
+        experts.apply(output, inp.hidden_states, inp.w1, inp.w2, inp.topk_weights, inp.topk_ids, activation="silu",
+                      global_num_experts=inp.w1.shape[0], expert_map=None, a1q_scale=None, a2_scale=None,
+                      workspace13=junk, workspace2=junk, expert_tokens_meta=None, apply_router_weight_on_input=False)
+        assert output.data_ptr() == before and torch.equal(output, plain)
+        assert rel_err(output, want) < TOL
+        with pytest.raises(NotImplementedError):
+            experts.apply(output, inp.hidden_states, inp.w1, inp.w2, inp.topk_weights, inp.topk_ids,
+                          expert_map=torch.arange(inp.w1.shape[0], device=DEV))
+        # in place: out is the input tensor
+        x = inp.hidden_states.clone()
+        ret = pra.fused_experts(x, *inp.fused_experts_args()[1:], out=x, **inp.fused_experts_kwargs())
+        assert ret is x and torch.equal(x, plain)
+        # wrong shape or dtype of out is refused before anything runs
+        with pytest.raises(ValueError):
+            pra.fused_experts(*inp.fused_experts_args(), out=out[:, :-8], **inp.fused_experts_kwargs())
+        with pytest.raises(ValueError):
+            pra.fused_experts(*inp.fused_experts_args(), out=out.float(), **inp.fused_experts_kwargs())
 
 
 # The LDS-tiled family builds its tile list inside the kernel; inside fused_experts (expert ids known to

@@ -167,3 +167,93 @@ def test_policy_update_hook_writes_layer_parameters_in_place(pra, oracle):
         pra.load_quantized_expert_weights(params, "model.layers.0.mlp.experts",
                                           *[t[:4].to(DEV) for t in new])
     assert torch.equal(got[0], snapshot)
+
+
+def test_model_level_weight_update_from_a_name_tensor_stream(pra, oracle):
+    """``load_weights_kernel_int8``, the int8 counterpart of the reference's ``load_weights_kernel``
+    (src/prime_rl/inference/vllm/worker/weight_transfer.py:97-134), on a two-layer stand-in model: one layer's
+    experts arrive under the trainer's names (gate_proj / up_proj / down_proj), the other's in kernel format
+    (bf16 w13_weight / w2_weight) and interleaved with other tensors; the engine nests one layer's parameters
+    under ``routed_experts`` and keeps the other flat.  Every parameter is rewritten at its address with the
+    oracle's bits; tensors that are not expert weights are copied; bad names and shapes are all reported in
+    ONE error after everything valid has been written."""
+    im = inputs_mod()
+    shape = im.SHAPES["toy"]
+    E, I, H = shape.E_total, shape.I, shape.H
+    names = ("w13_weight", "w13_weight_scale", "w2_weight", "w2_weight_scale")
+    params = {}
+    for layer, nested, seed in ((0, ".routed_experts", 30), (1, "", 31)):
+        old = pra.quantize_expert_weights(*[t.to(DEV) for t in _weights(E, I, H, seed=seed, spread=False)])
+        for name, t in zip(names, old):
+            if name.endswith("_scale") and layer == 0:
+                t = t.unsqueeze(-1).contiguous()
+            params[f"model.layers.{layer}.mlp.experts{nested}.{name}"] = torch.nn.Parameter(t, requires_grad=False)
+        params[f"model.layers.{layer}.input_layernorm.weight"] = torch.nn.Parameter(
+            torch.zeros(H, dtype=torch.bfloat16, device=DEV), requires_grad=False)
+    ptrs = {k: v.data_ptr() for k, v in params.items()}
+    new0 = _weights(E, I, H, seed=32, spread=False)
+    new1 = _weights(E, I, H, seed=33, spread=True)
+    norm = torch.randn(H, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+
+    def stream():
+        yield "model.layers.0.mlp.experts.gate_proj", new0[0].to(DEV)
+        yield "model.layers.1.mlp.experts.w2_weight", new1[2].to(DEV)           # kernel format, bf16 payload
+        yield "model.layers.0.input_layernorm.weight", norm.to(DEV)
+        yield "model.layers.0.mlp.experts.down_proj", new0[2].to(DEV)
+        yield "model.layers.1.mlp.experts.w13_weight", torch.cat([new1[0], new1[1]], dim=1).to(DEV)
+        yield "model.layers.0.mlp.experts.up_proj", new0[1].to(DEV)
+        yield "model.layers.1.input_layernorm.weight", (norm * 2).to(DEV)
+
+    class Model:  # enough of a module: named_parameters()
+        def named_parameters(self):
+            return iter(params.items())
+
+    result = pra.load_weights_kernel_int8(Model(), stream())
+    assert sorted(result["quantized_layers"]) == ["model.layers.0.mlp.experts", "model.layers.1.mlp.experts"]
+    assert sorted(result["loaded"]) == sorted(params)
+    assert {k: v.data_ptr() for k, v in params.items()} == ptrs
+    for layer, nested, new in ((0, ".routed_experts", new0), (1, "", new1)):
+        want = oracle.quantize_expert_weights(*new)
+        got = [params[f"model.layers.{layer}.mlp.experts{nested}.{n}"].cpu() for n in names]
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1].reshape(want[1].shape), want[1])
+        assert torch.equal(got[2], want[2]) and torch.equal(got[3].reshape(want[3].shape), want[3])
+    assert torch.equal(params["model.layers.0.input_layernorm.weight"].cpu(), norm)
+    assert torch.equal(params["model.layers.1.input_layernorm.weight"].cpu(), norm * 2)
+    # the layer computes with the new weights
+    x = torch.randn(24, H, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16)
+    tw, ids = im.route(shape, 24, torch.Generator().manual_seed(6))
+    l1 = [params[f"model.layers.1.mlp.experts.{n}"] for n in names]
+    out = pra.fused_experts(x.to(DEV), l1[0], l1[2], tw.to(DEV), ids.to(DEV), use_int8_w8a8=True,
+                            per_channel_quant=True, w1_scale=l1[1], w2_scale=l1[3])
+    want1 = oracle.quantize_expert_weights(*new1)
+    assert rel_err(out.cpu(), oracle.fused_experts(x, want1[0], want1[2], tw, ids, want1[1], want1[3])) < 1e-2
+
+    # a stream with several faults: everything valid is still written, one error names all the rest
+    newer = _weights(E, I, H, seed=34, spread=False)
+
+    def faulty():
+        yield "model.layers.1.mlp.experts.gate_proj", newer[0].to(DEV)
+        yield "model.layers.9.mlp.experts.gate_proj", newer[0].to(DEV)          # a layer the model does not have ...
+        yield "model.layers.9.mlp.experts.up_proj", newer[1].to(DEV)
+        yield "model.layers.9.mlp.experts.down_proj", newer[2].to(DEV)
+        yield "model.layers.0.mlp.experts.gate_proj", newer[0][:4].to(DEV)      # ... wrong expert count ...
+        yield "model.layers.0.mlp.experts.up_proj", newer[1][:4].to(DEV)
+        yield "model.layers.0.mlp.experts.down_proj", newer[2][:4].to(DEV)
+        yield "model.layers.1.mlp.experts.up_proj", newer[1].to(DEV)
+        yield "model.norm.weight", norm.to(DEV)                                  # ... an unknown plain tensor ...
+        yield "model.layers.0.input_layernorm.weight", norm[:-8].to(DEV)        # ... a plain tensor of the wrong shape
+        yield "model.layers.1.mlp.experts.down_proj", newer[2].to(DEV)
+        yield "model.layers.0.mlp.experts.w13_weight", torch.cat([newer[0], newer[1]], dim=1).to(DEV)  # never completed
+
+    layer0_before = params["model.layers.0.mlp.experts.routed_experts.w13_weight"].detach().clone()
+    with pytest.raises(ValueError) as err:
+        pra.load_weights_kernel_int8(params, faulty())
+    msg = str(err.value)
+    assert "shape mismatches" in msg and "not found in model" in msg
+    for fragment in ("model.layers.9.mlp.experts.w13_weight", "model.norm.weight", "model.layers.0.input_layernorm.weight",
+                     "model.layers.0.mlp.experts.routed_experts.w13_weight", "incomplete expert group"):
+        assert fragment in msg, fragment
+    assert torch.equal(params["model.layers.0.mlp.experts.routed_experts.w13_weight"], layer0_before)
+    want = oracle.quantize_expert_weights(*newer)
+    assert torch.equal(params["model.layers.1.mlp.experts.w13_weight"].cpu(), want[0])   # the valid layer was written
+    assert {k: v.data_ptr() for k, v in params.items()} == ptrs

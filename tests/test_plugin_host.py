@@ -260,3 +260,61 @@ def test_pinned_workspaces_are_never_freed(pra, monkeypatch):
         api._workspace(dev, stream, 64)
     assert api._workspaces[(0, 9)] is pinned
     assert len(api._workspaces) <= api._MAX_CACHED_WORKSPACES
+
+
+def test_experts_selection_hook(pra, monkeypatch):
+    """``register_experts_selection`` against a stand-in quantisation-method class: gated by the environment,
+    idempotent, returns the HIP experts for an eligible layer and defers to the original for an expert map, static
+    activation scales, another dtype, or a shape the kernels do not take."""
+    vp = pra.vllm_plugin
+    module_name, class_name = vp.MODULAR_METHODS[0]
+    parts = module_name.split(".")
+    for i in range(1, len(parts) + 1):
+        name = ".".join(parts[:i])
+        if name not in sys.modules:
+            monkeypatch.setitem(sys.modules, name, types.ModuleType(name))
+
+    class Method:
+        static_input_scales = False
+
+        def select_gemm_impl(self, prepare_finalize, layer):
+            return "original experts"
+
+    monkeypatch.setattr(sys.modules[module_name], class_name, Method, raising=False)
+
+    def layer(**over):
+        base = dict(w13_weight=torch.empty(4, 256, 128, dtype=torch.int8, device="meta"),
+                    w2_weight=torch.empty(4, 128, 128, dtype=torch.int8, device="meta"),
+                    w13_weight_scale="s13", w2_weight_scale="s2", expert_map=None, activation="silu")
+        base.update(over)
+        return types.SimpleNamespace(**base)
+
+    monkeypatch.delenv(vp.ENV_FLAG, raising=False)
+    assert vp.register_experts_selection() is False
+    assert Method().select_gemm_impl(None, layer()) == "original experts"
+    monkeypatch.setenv(vp.ENV_FLAG, "1")
+    assert vp.register_experts_selection() is True
+    assert vp.register_experts_selection() is False  # the marker: nothing is wrapped twice
+    experts = Method().select_gemm_impl("prepare/finalize", layer())
+    assert isinstance(experts, vp.Int8W8A8HipExperts) and experts.w1_scale == "s13" and experts.w2_scale == "s2"
+    for other in (dict(expert_map=torch.arange(4)), dict(activation="gelu"), dict(w13_input_scale=torch.ones(1)),
+                  dict(w13_weight=torch.empty(4, 256, 128, dtype=torch.float8_e4m3fn, device="meta")),
+                  dict(w13_weight=torch.empty(4, 200, 128, dtype=torch.int8, device="meta")),
+                  dict(w2_weight_scale=None)):
+        assert Method().select_gemm_impl(None, layer(**other)) == "original experts", other
+    static = Method()
+    static.static_input_scales = True
+    assert static.select_gemm_impl(None, layer()) == "original experts"
+    # another quantisation method can be named through the environment
+    other_mod = types.ModuleType("vllm_standin_quant")
+
+    class Other(Method):
+        pass
+
+    Other.select_gemm_impl = lambda self, prepare_finalize, layer: "other original"
+    other_mod.Other = Other
+    monkeypatch.setitem(sys.modules, "vllm_standin_quant", other_mod)
+    monkeypatch.setenv(vp.ENV_METHODS, "vllm_standin_quant:Other")
+    assert vp.register_experts_selection() is True
+    assert isinstance(Other().select_gemm_impl(None, layer()), vp.Int8W8A8HipExperts)
+    assert Other().select_gemm_impl(None, layer(expert_map="map")) == "other original"
