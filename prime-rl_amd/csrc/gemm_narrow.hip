@@ -97,6 +97,16 @@ __device__ __forceinline__ void load_to_lds_16(const void* base, uint32_t offset
                : "s"((uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(offset), "s"(uniform_address(base))
                : "memory", "m0");
 }
+// The same with the non-temporal hint: for weight rows that no other tile of this launch reads (the
+// expert's rows fit in one tile).  Streamed that way they do not displace the token rows and the
+// other tiles' shared weights from L2: measured 8-13 % on launches bound by the weight stream, and
+// a loss wherever a second tile of the expert would have found the rows in L2, hence per task.
+__device__ __forceinline__ void load_to_lds_16_stream(const void* base, uint32_t offset, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+               :
+               : "s"((uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(offset), "s"(uniform_address(base))
+               : "memory", "m0");
+}
 __device__ __forceinline__ void load_to_lds_4(const void* base, uint32_t offset, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
                :
@@ -126,10 +136,12 @@ struct Task {
   int e;          // expert; -1 = no more work
   int ct;         // channel tile
   int64_t slot0;  // first slot of the tile in sorted_ids
+  bool single;    // the expert's rows fit in this one tile: nothing else reads its weight rows
 };
 
 struct TaskLoads {
   const int8_t* wbase;  // weights of the task's expert (wave-uniform)
+  bool stream;          // fetch the weight rows with the non-temporal hint
   uint32_t woff[4];     // per lane: byte offset of its chunk of weight row i from wbase
   uint32_t xoff[2];     // per lane: byte offset of its chunk of token row i from a_q
 };
@@ -185,6 +197,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_narrow_kernel(NarrowParams p
     tk.e = -1;
     tk.ct = 0;
     tk.slot0 = 0;
+    tk.single = false;
     for (; xcd * per_xcd + it < range_end; it += stride) {
       const int task = xcd * per_xcd + it;
       const int tile = task / p.ntiles;
@@ -196,6 +209,24 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_narrow_kernel(NarrowParams p
         tk.e = e;
         tk.ct = task - tile * p.ntiles;
         tk.slot0 = slot0;
+        // Does the expert hold other tiles?  Its neighbours in the block list, and the other
+        // 64-row half of a 128-row block (valid rows are a prefix: a second half means the first is
+        // full, and the second half's first slot says whether it is in use).
+        const int nblocks = npp / p.B;
+        int32_t before, after;
+        scalar_load2(p.expert_ids + (blk > 0 ? blk - 1 : blk), p.expert_ids + (blk + 1 < nblocks ? blk + 1 : blk), before,
+                     after);
+        bool single = (blk == 0 || before != e) && (blk + 1 >= nblocks || after != e);
+        if (single && sub_per_block > 1) {
+          if (tile % sub_per_block != 0) {
+            single = false;
+          } else {
+            int32_t other, unused;
+            scalar_load2(p.sorted_ids + slot0 + kTok, p.sorted_ids + slot0, other, unused);
+            single = !(other >= 0 && other < p.P);
+          }
+        }
+        tk.single = single;
         break;
       }
     }
@@ -224,6 +255,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_narrow_kernel(NarrowParams p
       ld.woff[i] = (uint32_t)n * (uint32_t)K + chunk;
     }
     ld.wbase = p.w + (int64_t)tk.e * p.N * K;
+    ld.stream = tk.single;
   };
   auto setup_token_loads = [&](const TileAux& ax, TaskLoads& ld) {
 #pragma unroll
@@ -237,8 +269,13 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_narrow_kernel(NarrowParams p
   };
   auto issue_weights = [&](const TaskLoads& ld, int stage, int koff) {
     const uint32_t base = stage0 + stage * kStageBytes;
+    if (ld.stream) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) load_to_lds_16(ld.wbase + koff, ld.woff[i], base + (wave * 4 + i) * 1024);
+      for (int i = 0; i < 4; ++i) load_to_lds_16_stream(ld.wbase + koff, ld.woff[i], base + (wave * 4 + i) * 1024);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) load_to_lds_16(ld.wbase + koff, ld.woff[i], base + (wave * 4 + i) * 1024);
+    }
   };
   auto issue_tokens = [&](const TaskLoads& ld, int stage, int koff) {
     const uint32_t base = stage0 + stage * kStageBytes + kTokOffset;

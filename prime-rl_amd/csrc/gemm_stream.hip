@@ -161,9 +161,10 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
     const int wave = threadIdx.x / kWave;
     const int row_bytes = K + kFusedRowPad;
     __syncthreads();  // the previous pass is done reading a_lds
+    // valid rows are a prefix of the sub-tile: dealt round-robin, the wavefronts share them evenly
 #pragma unroll
     for (int i = 0; i < kSub / kWaves; ++i) {
-      const int r = wave * (kSub / kWaves) + i;
+      const int r = i * kWaves + wave;
       const int32_t t = p.sorted_ids[(int64_t)blk * p.B + sub0 * kSub + r];  // wave-uniform
       if (t < 0 || t >= p.P) continue;
       const uint4* in = reinterpret_cast<const uint4*>(p.a_bf16 + (int64_t)t * K);
