@@ -50,7 +50,13 @@ int check_gemm_common(const void* a_q, const void* w, const int32_t* sorted, con
   return MOE_I8_OK;
 }
 
-constexpr int kStreamRowsPerExpert = 8;
+// The streaming family reads an expert's weights once per 16 of its rows: it is the fastest kernel
+// while every block fits one such pass, and loses badly as soon as a few experts hold more (a
+// shared expert that every token visits, skewed routing), which the host cannot see.  It is
+// therefore picked where no expert can hold more than 16 rows (it holds at most one per token),
+// or where there is at most one routed row per expert on average.
+constexpr int kStreamMaxRows = 16;
+constexpr int kStreamRowsPerExpert = 1;
 
 int tile_geometry_of(int variant) {
   return variant == MOE_I8_GEMM_TILE_WIDE ? moe_i8::kTileWide
@@ -62,11 +68,11 @@ int tile_geometry_of(int variant) {
 // The narrow tiles (two small workgroups per compute unit, 64 x 128 tasks) start up faster and
 // balance better; the deep tiles stream an expert's weights once for up to 128 rows, which counts
 // the more the longer a launch runs and the more the routing is skewed.  Measured crossovers, with
-// the weight bytes of the launch: 0.2-0.4 GB (Qwen3-30B-A3B, even routing) 32-48 rows, 0.7-1.5 GB
-// (GLM-4.5-Air, Zipf routing and a shared expert) 24-32, 3.8-7.5 GB (DeepSeek-V3) below 8.
+// the weight bytes of the launch: 0.2-0.4 GB (Qwen3-30B-A3B, even routing) 40 rows, 0.7-1.5 GB
+// (GLM-4.5-Air, Zipf routing and a shared expert) 24-32, 3.8-7.5 GB (DeepSeek-V3) about 8.
 int narrow_rows_per_expert(const moe_i8::GemmArgs& g) {
   const int64_t weight_bytes = (int64_t)g.num_experts * g.n * g.k;
-  return weight_bytes < (512ll << 20) ? 44 : weight_bytes < (2048ll << 20) ? 24 : 8;
+  return weight_bytes < (512ll << 20) ? 40 : weight_bytes < (2048ll << 20) ? 28 : 8;
 }
 
 // Which family a launch goes to (MOE_I8_GEMM_STREAM, _TILE or _NARROW); -1 with the error set if a
@@ -85,15 +91,16 @@ int picks_family(const moe_i8::GemmArgs& g0, int variant) {
     return MOE_I8_GEMM_NARROW;
   }
   if (variant == MOE_I8_GEMM_STREAM) return MOE_I8_GEMM_STREAM;
-  // Measured crossovers, in routed rows per expert.  With evenly spread routing the streaming
-  // family wins while a block mostly holds one 16-row sub-tile (up to about 12); it reads an
-  // expert's weights once per 16 (or 32) of its rows, so skewed routing costs it far more than the
-  // tiled families (a few experts with a hundred rows double its time), and the first crossover is
-  // therefore set lower, at 8, where the narrow tiles lose 2 % or less on even routing.  Then the
-  // narrow tiles while most experts hold a single 64-row block, then the LDS-tiled family (which
-  // picks its own geometry).
+  // Measured crossovers, in routed rows per expert.  With evenly spread routing the streaming family
+  // would win up to about 4 (by 1-2 % over the narrow tiles); with one expert that every token visits,
+  // or Zipf-skewed routing, the narrow tiles win by 18-34 % from 24 tokens on.  Then the narrow tiles
+  // while most experts hold a single 64-row block, then the LDS-tiled family (which picks its own
+  // geometry).
   const int64_t rows_x_experts = g.num_pairs;
-  if (rows_x_experts <= (int64_t)kStreamRowsPerExpert * g.num_experts) return MOE_I8_GEMM_STREAM;
+  const int64_t most_rows = g.max_rows_per_expert > 0 && g.max_rows_per_expert < g.num_pairs ? g.max_rows_per_expert
+                                                                                             : g.num_pairs;
+  if (most_rows <= kStreamMaxRows || rows_x_experts <= (int64_t)kStreamRowsPerExpert * g.num_experts)
+    return MOE_I8_GEMM_STREAM;
   if (rows_x_experts <= (int64_t)narrow_rows_per_expert(g) * g.num_experts && moe_i8::gemm_narrow_supports(g))
     return MOE_I8_GEMM_NARROW;
   if (moe_i8::gemm_tile_supports(g)) return MOE_I8_GEMM_TILE;

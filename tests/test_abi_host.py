@@ -221,16 +221,20 @@ _PLAN = [
     ("toy", 256, "tile_deep", "tile_deep", 5),
     ("qwen3-30b-a3b", 1, "stream", "stream", 4),
     ("qwen3-30b-a3b", 16, "stream", "stream", 4),
-    ("qwen3-30b-a3b", 128, "stream", "stream", 5),
+    ("qwen3-30b-a3b", 17, "narrow", "narrow", 5),   # more than 16 tokens: a block may need a second streaming pass
+    ("qwen3-30b-a3b", 128, "narrow", "narrow", 5),
     ("qwen3-30b-a3b", 256, "narrow", "narrow", 5),
     ("qwen3-30b-a3b", 512, "narrow", "narrow", 5),
+    ("qwen3-30b-a3b", 640, "narrow", "narrow", 5),
+    ("qwen3-30b-a3b", 704, "tile_deep", "tile_deep", 5),
     ("qwen3-30b-a3b", 1024, "tile_deep", "tile_deep", 5),
     ("qwen3-30b-a3b", 8192, "tile_wide", "tile_wide", 7),
-    ("glm-4.5-air", 32, "stream", "stream", 5),
+    ("glm-4.5-air", 16, "stream", "stream", 5),
+    ("glm-4.5-air", 32, "narrow", "narrow", 5),     # the shared expert holds every token: 32 rows in one block
     ("glm-4.5-air", 512, "tile_deep", "tile_deep", 5),
     ("glm-4.5-air", 4096, "tile_wide", "tile_wide", 7),
     ("deepseek-v3", 8, "stream", "stream", 5),
-    ("deepseek-v3", 64, "stream", "stream", 5),
+    ("deepseek-v3", 64, "narrow", "narrow", 5),
     ("deepseek-v3", 2048, "tile_deep", "tile_deep", 6),
     ("deepseek-v3", 16384, "tile_wide", "tile_wide", 7),
 ]
