@@ -141,7 +141,8 @@ def time_stages(pkg, torch, shape, dev, weights, steps: int, warmup: int, varian
     tw = dev.topk_weights.reshape(-1).contiguous()
     stream = torch.cuda.current_stream().cuda_stream
     v = {"auto": abi.GEMM_AUTO, "stream": abi.GEMM_STREAM, "tile": abi.GEMM_TILE, "narrow": abi.GEMM_NARROW,
-         "tile_wide": abi.GEMM_TILE_WIDE, "tile_deep": abi.GEMM_TILE_DEEP}[variant]
+         "tile_wide": abi.GEMM_TILE_WIDE, "tile_deep": abi.GEMM_TILE_DEEP,
+         "tile_ring": abi.GEMM_TILE_RING}[variant]
     n = len(weights)
     p_ = lambda t: t.data_ptr()
     stages = [
@@ -540,7 +541,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--m", type=int, default=8192, help="tokens per step of the headline measurement")
     ap.add_argument("--shape", default="qwen3-30b-a3b")
-    ap.add_argument("--variant", default="auto", choices=["auto", "stream", "tile", "narrow", "tile_wide", "tile_deep"])
+    ap.add_argument("--variant", default="auto", choices=["auto", "stream", "tile", "narrow", "tile_wide", "tile_deep", "tile_ring"])
     ap.add_argument("--weight-copies", type=int, default=4)
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")

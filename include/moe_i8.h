@@ -44,6 +44,8 @@ extern "C" {
 #define MOE_I8_GEMM_NARROW 3 /* 64-row tiles, three LDS stages kept in flight (tens of rows per expert) */
 #define MOE_I8_GEMM_TILE_WIDE 4 /* the LDS-tiled family with 256-row tiles and two stages (many rows per expert) */
 #define MOE_I8_GEMM_TILE_DEEP 5 /* the LDS-tiled family with 128-row tiles and three stages (around 100 rows per expert) */
+#define MOE_I8_GEMM_TILE_RING 6 /* 256-row tiles through a ring of four 32 KB stages: a measured alternative to _TILE_WIDE, \
+                                   same results, 7-10 % slower; MOE_I8_GEMM_AUTO never picks it */
 
 /* Router score functions (reference TokenChoiceTopKRouter.score_func). */
 #define MOE_I8_SCORE_SOFTMAX 0      /* softmax over all experts */

@@ -17,7 +17,7 @@ PROBE_LIB_PATH = PKG_DIR / "libmoe_i8_probe.so"  # benchmark aid, not part of th
 OK = 0
 EINVAL, EWORKSPACE, ELAUNCH, EUNSUPPORTED = -1, -2, -3, -4
 DTYPE_BF16 = 0
-GEMM_AUTO, GEMM_STREAM, GEMM_TILE, GEMM_NARROW, GEMM_TILE_WIDE, GEMM_TILE_DEEP = 0, 1, 2, 3, 4, 5
+GEMM_AUTO, GEMM_STREAM, GEMM_TILE, GEMM_NARROW, GEMM_TILE_WIDE, GEMM_TILE_DEEP, GEMM_TILE_RING = 0, 1, 2, 3, 4, 5, 6
 SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_TOPK_SOFTMAX = 0, 1, 2
 MAX_EXPERTS = 1024
 

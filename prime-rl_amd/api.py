@@ -48,7 +48,7 @@ __all__ = [
 DEFAULT_BLOCK_SIZE_M = 64
 _VARIANTS = {
     "auto": _abi.GEMM_AUTO, "stream": _abi.GEMM_STREAM, "tile": _abi.GEMM_TILE, "narrow": _abi.GEMM_NARROW,
-    "tile_wide": _abi.GEMM_TILE_WIDE, "tile_deep": _abi.GEMM_TILE_DEEP,
+    "tile_wide": _abi.GEMM_TILE_WIDE, "tile_deep": _abi.GEMM_TILE_DEEP, "tile_ring": _abi.GEMM_TILE_RING,
 }
 # Default workspaces, one per (device, stream) that has called without a caller-owned one: a small
 # LRU (a process has a handful of forward streams) guarded by a lock.  Entries are only ever created or
@@ -115,7 +115,7 @@ def workspace_bytes(m: int, top_k: int, num_experts: int, hidden: int, inter: in
 
 
 _KERNEL_NAMES = {_abi.GEMM_STREAM: "stream", _abi.GEMM_NARROW: "narrow", _abi.GEMM_TILE_WIDE: "tile_wide",
-                 _abi.GEMM_TILE_DEEP: "tile_deep"}
+                 _abi.GEMM_TILE_DEEP: "tile_deep", _abi.GEMM_TILE_RING: "tile_ring"}
 
 
 def layer_plan(m: int, top_k: int, num_experts: int, hidden: int, inter: int,

@@ -45,7 +45,7 @@ int check_gemm_common(const void* a_q, const void* w, const int32_t* sorted, con
   if (k < 64 || k % 64) return fail(MOE_I8_EINVAL, "reduction length (%d) must be a positive multiple of 64", k);
   if (sorted_cap < moe_i8_sorted_capacity(num_pairs, num_experts, block_size))
     return fail(MOE_I8_EWORKSPACE, "sorted_token_ids capacity %lld too small", (long long)sorted_cap);
-  if (variant < MOE_I8_GEMM_AUTO || variant > MOE_I8_GEMM_TILE_DEEP)
+  if (variant < MOE_I8_GEMM_AUTO || variant > MOE_I8_GEMM_TILE_RING)
     return fail(MOE_I8_EINVAL, "unknown GEMM variant %d", variant);
   return MOE_I8_OK;
 }
@@ -61,6 +61,7 @@ constexpr int kStreamRowsPerExpert = 1;
 int tile_geometry_of(int variant) {
   return variant == MOE_I8_GEMM_TILE_WIDE ? moe_i8::kTileWide
          : variant == MOE_I8_GEMM_TILE_DEEP ? moe_i8::kTileDeep
+         : variant == MOE_I8_GEMM_TILE_RING ? moe_i8::kTileRing
                                             : moe_i8::kTileAuto;
 }
 
@@ -80,7 +81,8 @@ int narrow_rows_per_expert(const moe_i8::GemmArgs& g) {
 int picks_family(const moe_i8::GemmArgs& g0, int variant) {
   moe_i8::GemmArgs g = g0;
   g.tile_geometry = tile_geometry_of(variant);
-  if (variant == MOE_I8_GEMM_TILE || variant == MOE_I8_GEMM_TILE_WIDE || variant == MOE_I8_GEMM_TILE_DEEP) {
+  if (variant == MOE_I8_GEMM_TILE || variant == MOE_I8_GEMM_TILE_WIDE || variant == MOE_I8_GEMM_TILE_DEEP ||
+      variant == MOE_I8_GEMM_TILE_RING) {
     if (!moe_i8::gemm_tile_supports(g))
       return fail(MOE_I8_EUNSUPPORTED, "tile GEMM does not support this shape"), -1;
     return MOE_I8_GEMM_TILE;
@@ -146,13 +148,17 @@ moe_i8::GemmArgs gate_up_args(const int8_t* x_q, const float* a_scale, const int
 }
 
 // The family of `picks_family` with the geometry of the LDS-tiled family spelled out
-// (MOE_I8_GEMM_STREAM, _NARROW, _TILE_WIDE or _TILE_DEEP); -1 as there.
+// (MOE_I8_GEMM_STREAM, _NARROW, _TILE_WIDE or _TILE_DEEP; _TILE_RING only when demanded); -1 as there.
 int picks_kernel(const moe_i8::GemmArgs& g0, int variant) {
   const int family = picks_family(g0, variant);
   if (family != MOE_I8_GEMM_TILE) return family;
   moe_i8::GemmArgs g = g0;
   g.tile_geometry = tile_geometry_of(variant);
-  return moe_i8::gemm_tile_geometry(g) == moe_i8::kTileDeep ? MOE_I8_GEMM_TILE_DEEP : MOE_I8_GEMM_TILE_WIDE;
+  switch (moe_i8::gemm_tile_geometry(g)) {
+    case moe_i8::kTileDeep: return MOE_I8_GEMM_TILE_DEEP;
+    case moe_i8::kTileRing: return MOE_I8_GEMM_TILE_RING;
+    default: return MOE_I8_GEMM_TILE_WIDE;
+  }
 }
 
 moe_i8::GemmArgs down_args(const int8_t* h_q, const float* a_scale, const int8_t* w2, const float* w2_scale,
@@ -662,7 +668,7 @@ int moe_i8_layer_plan(int64_t m, int top_k, int num_experts, int hidden_size, in
   if (!valid_block_size(block_size)) return fail(MOE_I8_EINVAL, "block_size must be 16, 32, 64 or 128");
   if (hidden_size < 64 || hidden_size % 64 || inter < 64 || inter % 64)
     return fail(MOE_I8_EINVAL, "hidden (%d) and inter (%d) must be positive multiples of 64", hidden_size, inter);
-  if (variant < MOE_I8_GEMM_AUTO || variant > MOE_I8_GEMM_TILE_DEEP)
+  if (variant < MOE_I8_GEMM_AUTO || variant > MOE_I8_GEMM_TILE_RING)
     return fail(MOE_I8_EINVAL, "unknown GEMM variant %d", variant);
   const LayerPlan plan = plan_layer(m, top_k, num_experts, hidden_size, inter, block_size, variant);
   if (plan.gate_up_kernel < 0 || plan.down_kernel < 0) return MOE_I8_EUNSUPPORTED;

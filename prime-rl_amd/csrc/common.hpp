@@ -221,9 +221,9 @@ struct GemmArgs {
   void* out;  // bf16 [P, I] | bf16 [P, H] | int32 [P, N]
   int64_t max_rows_per_expert = 0;  // upper bound if the caller knows one (the token count), else 0
   bool expert_ids_ascend = false;   // expert_ids is known to come from moe_align (non-decreasing over the used blocks)
-  int tile_geometry = 0;            // LDS-tiled family: kTileAuto, kTileWide (256-row tiles) or kTileDeep (128-row tiles)
+  int tile_geometry = 0;            // LDS-tiled family: kTileAuto, kTileWide (256-row tiles), kTileDeep (128-row tiles) or kTileRing (256-row tiles, four-stage ring; on demand only)
 };
-constexpr int kTileAuto = 0, kTileWide = 1, kTileDeep = 2;
+constexpr int kTileAuto = 0, kTileWide = 1, kTileDeep = 2, kTileRing = 3;
 constexpr int kTileDeepRowsPerExpert = 96;  // the LDS-tiled family picks its deep geometry up to this many routed rows per expert
 hipError_t launch_gemm_stream(const GemmArgs& a, hipStream_t stream);
 // register-only int8 MFMA loop (measurement aid): sink holds mfma_probe_sink_bytes(workgroups)
@@ -234,7 +234,7 @@ bool gemm_stream_fuses_quant(int k);  // the down GEMM can quantise bf16 activat
 hipError_t launch_gemm_tile(const GemmArgs& a, hipStream_t stream);
 bool gemm_tile_supports(const GemmArgs& a);
 bool gemm_tile_prefers_deep(const GemmArgs& a);
-int gemm_tile_geometry(const GemmArgs& a);  // kTileWide or kTileDeep: what a launch of the family would use
+int gemm_tile_geometry(const GemmArgs& a);  // kTileWide or kTileDeep (kTileRing on demand): what a launch of the family would use
 hipError_t launch_gemm_narrow(const GemmArgs& a, hipStream_t stream);
 bool gemm_narrow_supports(const GemmArgs& a);
 

@@ -720,7 +720,397 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tile_kernel(TileParams p) {
     run(std::true_type{});
 }
 
-template <int MODE, bool DEEP>
+// ---------------------------------------------------------------------------------------------
+// Ring pipeline for the 256 x 256 tile (the geometry kTileRing; never chosen by itself, kept as a
+// measured alternative to the two-stage pipeline above): reduction steps of 64 bytes through a ring
+// of four 32 KB stages (16 KB of weight rows, then 16 KB of token rows), every stage filled three
+// steps before it is multiplied, so that up to 96 KB of loads are in flight per compute unit
+// against the 64 KB of the two-stage pipeline.  LDS rows are 64 bytes (four 16-byte chunks); a
+// wave-level load covers 16 rows.
+//
+// One barrier per step, placed in the MIDDLE of the step: the operands of the step's second
+// 32-byte half are read while the first half multiplies; once they are in registers the whole
+// stage has been consumed, so the barrier both frees it for the loads four steps ahead and
+// publishes the next stage, whose first-half operands are then read while the second half
+// multiplies.  The matrix pipe therefore always has eight MFMAs with their operands in registers
+// on either side of the barrier.
+//
+// Measured against the two-stage pipeline on 65536 routed rows x 128 experts (gate_up 4096 x 2048,
+// down 2048 x 2048): same results bit for bit, 7-10 % slower.  A lane's 16-byte load takes a
+// quarter of a 64-byte row, so every 128-byte line is requested from L2 twice (the request count
+// per launch doubles, the bytes fetched from HBM stay), and the path from L2 into LDS, not the
+// depth of the pipeline, is what bounds the loads of this tile.
+constexpr int kRingBK = 64;
+constexpr int kRingSlots = 4;
+constexpr int kRingHalf = kBN * kRingBK;    // 16 KB
+constexpr int kRingStage = 2 * kRingHalf;   // 32 KB
+constexpr int kRingLoads = 4;               // wave-level loads per wavefront and step
+
+// chunk swizzle of a 64-byte LDS row: 16 consecutive rows reading one logical chunk, and 8 rows
+// reading two neighbouring chunks, both spread over all banks
+__device__ __forceinline__ int swizzle_of_row64(int r) { return (((r >> 2) & 1) << 1) | ((r >> 3) & 1); }
+
+struct RingLoads {
+  const int8_t* wbase;
+  uint32_t woff[2];
+  uint32_t xoff[2];
+};
+
+// lane fills slot (lane & 3) of row 32 * wave + 16 * i + (lane >> 2) of the weight half and of the token half
+template <int MODE>
+__device__ __forceinline__ void ring_setup_loads(const TileParams& p, const Task& tk, int wave, int lane, RingLoads& ld) {
+  const int K = p.K;
+  const int inter = p.N / 2;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = 32 * wave + 16 * i + (lane >> 2);
+    const int chunk = ((lane & 3) ^ swizzle_of_row64(row)) * 16;
+    int n;
+    if constexpr (MODE == kGateUpSilu) {
+      const int ch = tk.nt * 128 + (row & 127);
+      n = (ch < inter ? ch : inter - 1) + (row >= 128 ? inter : 0);
+    } else {
+      const int ch = tk.nt * kBN + row;
+      n = ch < p.N ? ch : p.N - 1;
+    }
+    ld.woff[i] = (uint32_t)n * (uint32_t)K + chunk;
+    uint32_t arow = 0;
+    if ((row >> 6) < tk.nsub) {
+      const int32_t tok = p.sorted_ids[tk.slot0 + row];
+      if (tok >= 0 && tok < p.P) arow = (uint32_t)(tok / p.row_div);
+    }
+    ld.xoff[i] = arow * (uint32_t)K + chunk;
+  }
+  ld.wbase = p.w + (int64_t)tk.e * p.N * K;
+}
+
+__device__ __forceinline__ void ring_issue_loads(const RingLoads& ld, const int8_t* a_q, uint32_t stage_addr, int wave,
+                                                 int koff) {
+#pragma unroll
+  for (int i = 0; i < 2; ++i) load_to_lds_16(a_q + koff, ld.xoff[i], stage_addr + kRingHalf + (wave * 2 + i) * 1024);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) load_to_lds_16(ld.wbase + koff, ld.woff[i], stage_addr + (wave * 2 + i) * 1024);
+}
+
+struct RingReads {
+  int w_ld[4];
+  int x_ld[2];
+  int chunk[2];
+};
+
+struct RingOperands {
+  v4i a[4], b[2];
+};
+
+__device__ __forceinline__ void ring_read(const RingReads& rd, const char* stage, int kk, RingOperands& o) {
+  o.b[0] = *reinterpret_cast<const v4i*>(stage + rd.x_ld[0] + rd.chunk[kk]);
+  o.a[0] = *reinterpret_cast<const v4i*>(stage + rd.w_ld[0] + rd.chunk[kk]);
+  o.b[1] = *reinterpret_cast<const v4i*>(stage + rd.x_ld[1] + rd.chunk[kk]);
+#pragma unroll
+  for (int ci = 1; ci < 4; ++ci) o.a[ci] = *reinterpret_cast<const v4i*>(stage + rd.w_ld[ci] + rd.chunk[kk]);
+}
+
+__device__ __forceinline__ void ring_multiply(const RingOperands& o, v16i (&acc)[4][2]) {
+#pragma unroll
+  for (int ci = 0; ci < 4; ++ci)
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) acc[ci][tj] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.a[ci], o.b[tj], acc[ci][tj], 0, 0, 0);
+}
+
+__device__ __forceinline__ void wait_lds_reads() { __builtin_amdgcn_s_waitcnt(0xC07F); }  // lgkmcnt(0), others free
+
+// The epilogue of the ring pipeline: the same arithmetic as `epilogue` with four MFMA tiles per
+// wavefront, staged through 4 KB per wavefront (32 token rows x 64 channels of bf16 at a time).
+template <int MODE>
+__device__ __forceinline__ void ring_epilogue(const TileParams& p, const Task& tk, int wave, int lane, v16i (&acc)[4][2],
+                                              char* wave_lds, float* wave_scales) {
+  const int tg = wave / 2;
+  const int cpart = wave % 2;
+  const int lrow = lane & 31;
+  const int lhalf = lane >> 5;
+  const int inter = p.N / 2;
+  int32_t tok[2];
+#pragma unroll
+  for (int tj = 0; tj < 2; ++tj) {
+    tok[tj] = p.sorted_ids[tk.slot0 + tg * 64 + tj * 32 + lrow];
+    if (tok[tj] < 0 || tok[tj] >= p.P) tok[tj] = -1;
+  }
+  if constexpr (MODE == kAccI32) {
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+      if (tok[tj] < 0) continue;
+      int32_t* out = static_cast<int32_t*>(p.out) + (int64_t)tok[tj] * p.N;
+#pragma unroll
+      for (int ci = 0; ci < 4; ++ci)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = tk.nt * kBN + cpart * 128 + ci * 32 + 8 * q + 4 * lhalf;
+          if (n < p.N)
+            *reinterpret_cast<v4i*>(out + n) =
+                v4i{acc[ci][tj][4 * q], acc[ci][tj][4 * q + 1], acc[ci][tj][4 * q + 2], acc[ci][tj][4 * q + 3]};
+        }
+    }
+  } else if constexpr (MODE == kDown) {
+    const float* wsc = p.w_scale + (int64_t)tk.e * p.N;
+    const int n0 = tk.nt * kBN + cpart * 128;  // first channel of this wavefront
+    // channel scales through LDS (see `epilogue`)
+    {
+      const int n = n0 + 2 * lane;
+      *reinterpret_cast<float2*>(wave_scales + 2 * lane) =
+          n < p.N ? *reinterpret_cast<const float2*>(wsc + n) : make_float2(0.0f, 0.0f);
+    }
+    float as[2], rw[2];
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+      as[tj] = tok[tj] >= 0 ? p.a_scale[tok[tj] / p.row_div] : 0.0f;
+      rw[tj] = tok[tj] >= 0 ? (p.row_weight ? p.row_weight[tok[tj]] : 1.0f) : 0.0f;
+    }
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        // 32 token rows x 64 channels (MFMA tiles 2h and 2h + 1)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          const int ci = 2 * h + c / 4;
+          const int q = c % 4;
+          const float4 ws = *reinterpret_cast<const float4*>(wave_scales + ci * 32 + 8 * q + 4 * lhalf);
+          const int v[4] = {acc[ci][tj][4 * q], acc[ci][tj][4 * q + 1], acc[ci][tj][4 * q + 2], acc[ci][tj][4 * q + 3]};
+          *reinterpret_cast<uint2*>(wave_lds + lrow * 128 + ((c ^ staging_swizzle<8>(lrow)) * 16) + lhalf * 8) =
+              down_epilogue4(v, as[tj], ws, rw[tj]);
+        }
+        // everything this wavefront has in flight is complete before its first stores, which
+        // are then the only vector-memory work still pending when the next tile starts
+        if (tj == 0 && h == 0) wait_vmcnt<0>();
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = r * 8 + lane / 8;
+          const int chunk = lane % 8;
+          const uint4 v = *reinterpret_cast<const uint4*>(wave_lds + row * 128 + ((chunk ^ staging_swizzle<8>(row)) * 16));
+          const int32_t t = __shfl(tok[tj], row);
+          const int n = n0 + h * 64 + chunk * 8;
+          if (t >= 0 && n < p.N)
+            __builtin_nontemporal_store(v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w},
+                                        reinterpret_cast<v4i*>(static_cast<uint16_t*>(p.out) + (int64_t)t * p.N + n));
+        }
+      }
+    }
+  } else {
+    const float* wsc = p.w_scale + (int64_t)tk.e * p.N;
+    const int n0 = tk.nt * 128 + cpart * 64;  // first gate channel of this wavefront
+    float as[2];
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) as[tj] = tok[tj] >= 0 ? p.a_scale[tok[tj] / p.row_div] : 0.0f;
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+      // 32 token rows x 64 activation channels
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        // gate rows sit in MFMA tile gi at 8 * gq, the matching up rows in tile gi + 2
+        const int gi = c / 4;
+        const int gq = c % 4;
+        const int ui = gi + 2;
+        const int n = n0 + c * 8 + 4 * lhalf;
+        const int ns = n < inter ? n : 0;
+        const float4 wg = *reinterpret_cast<const float4*>(wsc + ns);
+        const float4 wu = *reinterpret_cast<const float4*>(wsc + inter + ns);
+        const int g[4] = {acc[gi][tj][4 * gq], acc[gi][tj][4 * gq + 1], acc[gi][tj][4 * gq + 2], acc[gi][tj][4 * gq + 3]};
+        const int u[4] = {acc[ui][tj][4 * gq], acc[ui][tj][4 * gq + 1], acc[ui][tj][4 * gq + 2], acc[ui][tj][4 * gq + 3]};
+        *reinterpret_cast<uint2*>(wave_lds + lrow * 128 + ((c ^ staging_swizzle<8>(lrow)) * 16) + lhalf * 8) =
+            silu_mul_epilogue4(g, u, as[tj], wg, wu);
+      }
+      if (tj == 0) wait_vmcnt<0>();  // as in the down epilogue: only the stores below stay pending
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = r * 8 + lane / 8;
+        const int chunk = lane % 8;
+        const uint4 v = *reinterpret_cast<const uint4*>(wave_lds + row * 128 + ((chunk ^ staging_swizzle<8>(row)) * 16));
+        const int32_t t = __shfl(tok[tj], row);
+        const int n = n0 + chunk * 8;
+        if (t >= 0 && n < inter)
+          __builtin_nontemporal_store(v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w},
+                                      reinterpret_cast<v4i*>(static_cast<uint16_t*>(p.out) + (int64_t)t * inter + n));
+      }
+    }
+  }
+}
+
+template <int MODE>
+__global__ __launch_bounds__(kThreads, 1) void gemm_ring_kernel(TileParams p) {
+  constexpr int kMaxTiles = 6144;
+  __shared__ __align__(16) char stages[kRingSlots * kRingStage];
+  __shared__ uint32_t tile_desc[kMaxTiles];
+  __shared__ int wave_part[kWaves];
+  __shared__ __align__(16) float channel_scales[kWaves * 128];
+  __shared__ int total_tiles;
+
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int my_sub = wave / 2;  // token sub-block this wavefront multiplies
+  const int nk = p.K / kRingBK;
+
+  const int npp = *p.npp;
+  const int nblocks = npp / p.B;
+  const int sub_per_block = p.B / 64;
+  const int per_tile = 256 / p.B;  // 2 or 4 blocks
+  const int ntile =
+      p.ascend ? build_tile_list_ascending(p.expert_ids, nblocks, p.E, per_tile == 4 ? 2 : 1, reinterpret_cast<int*>(stages),
+                                           wave_part, tile_desc, &total_tiles, kMaxTiles)
+               : build_tile_list(p.expert_ids, nblocks, per_tile, reinterpret_cast<int*>(stages), wave_part, tile_desc,
+                                 &total_tiles, kMaxTiles);
+  const int total = ntile * p.ntiles;
+  const int per_xcd = (total + kXcds - 1) / kXcds;
+  const int xcd = blockIdx.x % kXcds;
+  const int stride = gridDim.x / kXcds;
+
+  const int lrow = lane & 31;
+  const int lhalf = lane >> 5;
+  RingReads rd;
+  {
+    const int cpart = wave % 2;
+#pragma unroll
+    for (int ci = 0; ci < 4; ++ci) {
+      int row;
+      if constexpr (MODE == kGateUpSilu)
+        row = (ci < 2 ? 0 : 128) + cpart * 64 + (ci & 1) * 32 + lrow;  // LDS rows 0..127 gate, 128..255 up
+      else
+        row = cpart * 128 + ci * 32 + lrow;
+      rd.w_ld[ci] = row * kRingBK;
+    }
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) rd.x_ld[tj] = kRingHalf + (my_sub * 64 + tj * 32 + lrow) * kRingBK;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) rd.chunk[kk] = ((2 * kk + lhalf) ^ swizzle_of_row64(lrow)) * 16;
+  }
+  const uint32_t stage0 = lds_address(stages);
+
+  auto decode = [&](int it) {
+    Task tk;
+    tk.e = -1;
+    tk.nt = 0;
+    tk.slot0 = 0;
+    tk.nsub = 0;
+    if (it < per_xcd && xcd * per_xcd + it < total) {
+      const int task = xcd * per_xcd + it;
+      const int tile0 = task / p.ntiles;
+      const uint32_t d0 = tile_desc[tile0];
+      const int first = tile0 - (int)((d0 >> 20) & 7u);
+      const int T = (int)((d0 >> 24) & 15u);
+      const int pos = task - first * p.ntiles;
+      const uint32_t d = tile_desc[first + pos % T];
+      tk.nt = pos / T;
+      const int blk = (int)(d & 0xffffu);
+      const int e = p.expert_ids[blk];
+      tk.slot0 = (int64_t)blk * p.B;
+      tk.nsub = (int)((d >> 16) & 15u) * sub_per_block;
+      tk.e = (e >= 0 && e < p.E) ? e : -2;
+    }
+    return tk;
+  };
+
+  int it = blockIdx.x / kXcds;
+  Task tk = decode(it);
+  while (tk.e == -2) tk = decode(it += stride);
+  if (tk.e < 0) return;
+  RingLoads ld;
+  ring_setup_loads<MODE>(p, tk, wave, lane, ld);
+  int slot = 0;  // stage of the step being multiplied
+  // the scratch of the tile list lived in the stage memory; the builder ends with a barrier
+#pragma unroll
+  for (int s = 0; s < kRingSlots - 1; ++s) ring_issue_loads(ld, p.a_q, stage0 + s * kRingStage, wave, s * kRingBK);
+
+  bool stores_pending = false;
+  bool first_task = true;
+  while (true) {
+    int nit = it + stride;
+    Task nx = decode(nit);
+    while (nx.e == -2) nx = decode(nit += stride);
+    RingLoads nld = ld;
+    if (nx.e >= 0) ring_setup_loads<MODE>(p, nx, wave, lane, nld);
+    const bool has_next = nx.e >= 0;
+    const bool active = my_sub < tk.nsub;
+
+    // Task start.  The loads of steps 0..2 were issued during the previous task (or above), and every
+    // wavefront has waited for its share of step 0 (at the previous task's last barrier; here for the
+    // first task).  The barrier also ends the epilogue's use of the stage that step 3 goes to.
+    if (first_task) wait_vmcnt<2 * kRingLoads>();
+    first_task = false;
+    __builtin_amdgcn_s_barrier();
+    {
+      int fill = slot + kRingSlots - 1;
+      if (fill >= kRingSlots) fill -= kRingSlots;
+      ring_issue_loads(ld, p.a_q, stage0 + fill * kRingStage, wave, (kRingSlots - 1) * kRingBK);
+    }
+    v16i acc[4][2];
+#pragma unroll
+    for (int ci = 0; ci < 4; ++ci)
+#pragma unroll
+      for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[ci][tj][r] = 0;
+    RingOperands o0, o1;
+    if (active) ring_read(rd, stages + slot * kRingStage, 0, o0);
+    for (int s = 0; s < nk; ++s) {
+      const char* stage = stages + slot * kRingStage;
+      if (active) {
+        ring_read(rd, stage, 1, o1);
+        ring_multiply(o0, acc);
+      }
+      // The loads of the following step (this task's, or the next task's step 0) have landed for this
+      // wavefront.  Behind them in the queue: the loads of the two steps after it, where they exist.  A
+      // wavefront that has just run an epilogue waited for everything there and has only stores pending
+      // in front of the loads it issued since: it lets them drain for two steps.
+      const bool follows = s + 1 < nk || has_next;
+      if (follows && !(stores_pending && s < 2)) {
+        const int later = has_next ? 2 : nk - 2 - s;
+        if (later >= 2)
+          wait_vmcnt<2 * kRingLoads>();
+        else if (later == 1)
+          wait_vmcnt<kRingLoads>();
+        else
+          wait_vmcnt<0>();
+      }
+      wait_lds_reads();  // this wavefront is done with the stage
+      __builtin_amdgcn_s_barrier();
+      int nslot = slot + 1 == kRingSlots ? 0 : slot + 1;
+      if (s + 1 < nk) {
+        // refill the stage just consumed with the step four ahead (the last step's stage is left to
+        // the epilogue; its loads are issued at the start of the next task)
+        const int ahead = s + kRingSlots;
+        if (ahead < nk)
+          ring_issue_loads(ld, p.a_q, stage0 + slot * kRingStage, wave, ahead * kRingBK);
+        else if (has_next)
+          ring_issue_loads(nld, p.a_q, stage0 + slot * kRingStage, wave, (ahead - nk) * kRingBK);
+        if (active) ring_read(rd, stages + nslot * kRingStage, 0, o0);
+      }
+      if (active) ring_multiply(o1, acc);
+      slot = nslot;
+    }
+    const int last = slot == 0 ? kRingSlots - 1 : slot - 1;
+    if (active)
+      ring_epilogue<MODE>(p, tk, wave, lane, acc, stages + last * kRingStage + wave * 4096, channel_scales + wave * 128);
+    stores_pending = active && MODE != kAccI32;
+    if (!has_next) break;
+    tk = nx;
+    ld = nld;
+    it = nit;
+  }
+  wait_vmcnt<0>();
+}
+
+bool ring_supports(const GemmArgs& a) {
+  const int64_t act_rows = (a.num_pairs + a.row_div - 1) / a.row_div;
+  if (!((a.block_size == 64 || a.block_size == 128) && a.k % kRingBK == 0 && a.k >= kRingSlots * kRingBK && a.n % 16 == 0 &&
+        (int64_t)a.n * a.k < (1ll << 32) && act_rows * a.k < (1ll << 32)))
+    return false;
+  const int64_t blocks = (a.sorted_cap + a.block_size - 1) / a.block_size;
+  const int per_tile = 256 / a.block_size;
+  const int64_t tiles = a.expert_ids_ascend ? (blocks + per_tile - 1) / per_tile + a.num_experts : blocks;
+  return tiles <= 6144 && blocks <= (int64_t)(kRingSlots * kRingStage / sizeof(int)) && blocks <= 65535;
+}
+
+template <int MODE, bool DEEP, bool RING = false>
 hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   TileParams p;
   p.a_q = a.a_q;
@@ -741,7 +1131,10 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   p.ascend = a.expert_ids_ascend && a.num_experts <= 2 * kThreads ? 1 : 0;
   p.out = a.out;
   const int grid = device_cu_count() / kXcds * kXcds;
-  hipLaunchKernelGGL((gemm_tile_kernel<MODE, DEEP>), dim3((unsigned)grid), dim3(kThreads), 0, stream, p);
+  if constexpr (RING)
+    hipLaunchKernelGGL((gemm_ring_kernel<MODE>), dim3((unsigned)grid), dim3(kThreads), 0, stream, p);
+  else
+    hipLaunchKernelGGL((gemm_tile_kernel<MODE, DEEP>), dim3((unsigned)grid), dim3(kThreads), 0, stream, p);
   return hipGetLastError();
 }
 
@@ -769,6 +1162,7 @@ bool gemm_tile_supports(const GemmArgs& a) {
   switch (a.tile_geometry) {
     case kTileWide: return geometry_supports<false>(a);
     case kTileDeep: return geometry_supports<true>(a);
+    case kTileRing: return ring_supports(a);
     default: return geometry_supports<false>(a) || geometry_supports<true>(a);
   }
 }
@@ -781,15 +1175,25 @@ bool gemm_tile_prefers_deep(const GemmArgs& a) {
   return a.num_pairs <= (int64_t)kTileDeepRowsPerExpert * a.num_experts;
 }
 
-// The geometry a launch of this family uses for `a` (kTileWide or kTileDeep).
+// The geometry a launch of this family uses for `a` (kTileWide or kTileDeep; kTileRing only on demand).
 int gemm_tile_geometry(const GemmArgs& a) {
   if (a.tile_geometry == kTileWide) return kTileWide;
   if (a.tile_geometry == kTileDeep) return kTileDeep;
+  if (a.tile_geometry == kTileRing) return kTileRing;
   return geometry_supports<true>(a) && (gemm_tile_prefers_deep(a) || !geometry_supports<false>(a)) ? kTileDeep : kTileWide;
 }
 
 hipError_t launch_gemm_tile(const GemmArgs& a, hipStream_t stream) {
-  if (gemm_tile_geometry(a) == kTileDeep) {
+  const int geometry = gemm_tile_geometry(a);
+  if (geometry == kTileRing) {
+    switch (a.mode) {
+      case kGateUpSilu: return launch_mode<kGateUpSilu, false, true>(a, stream);
+      case kDown: return launch_mode<kDown, false, true>(a, stream);
+      case kAccI32: return launch_mode<kAccI32, false, true>(a, stream);
+      default: return hipErrorInvalidValue;
+    }
+  }
+  if (geometry == kTileDeep) {
     switch (a.mode) {
       case kGateUpSilu: return launch_mode<kGateUpSilu, true>(a, stream);
       case kDown: return launch_mode<kDown, true>(a, stream);

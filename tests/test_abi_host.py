@@ -254,6 +254,9 @@ def test_layer_plan_follows_a_demanded_family_and_rejects_what_it_cannot_run(pra
         "gate_up": "stream", "down": "stream", "launches": 7}
     assert pra.layer_plan(1024, 8, 128, 2048, 768, gemm_variant="tile_wide")["gate_up"] == "tile_wide"
     assert pra.layer_plan(1024, 8, 128, 2048, 768, gemm_variant="tile")["gate_up"] == "tile_deep"
+    # the ring pipeline runs only where it is demanded
+    assert pra.layer_plan(8192, 8, 128, 2048, 768, gemm_variant="tile_ring") == {
+        "gate_up": "tile_ring", "down": "tile_ring", "launches": 7}
     with pytest.raises(abi.MoeI8Error) as e:  # the tiled families take blocks of 64 or 128 rows only
         pra.layer_plan(1024, 8, 128, 2048, 768, block_size=16, gemm_variant="tile_wide")
     assert e.value.code == abi.EUNSUPPORTED

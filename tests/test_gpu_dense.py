@@ -32,7 +32,7 @@ def test_scaled_quant_tie_vector_and_rows(pra, oracle):
         pra.scaled_int8_quant(x.to(DEV), scale=torch.ones(1, device=DEV))
 
 
-@pytest.mark.parametrize("variant", ["auto", "stream", "tile_wide", "tile_deep", "narrow"])
+@pytest.mark.parametrize("variant", ["auto", "stream", "tile_wide", "tile_deep", "tile_ring", "narrow"])
 @pytest.mark.parametrize("M,N,K", [(1, 64, 256), (7, 128, 512), (64, 1536, 2048), (200, 2048, 768), (1000, 512, 1024)])
 def test_linear_is_bit_exact(pra, oracle, variant, M, N, K):
     g = torch.Generator().manual_seed(M + N)
@@ -61,7 +61,7 @@ def test_linear_accepts_the_transposed_view_and_batched_input(pra, oracle):
         pra.apply_int8_linear(x.to(DEV)[..., :128].contiguous(), wd, s.to(DEV))
 
 
-@pytest.mark.parametrize("variant", ["auto", "stream", "tile_wide", "tile_deep", "narrow"])
+@pytest.mark.parametrize("variant", ["auto", "stream", "tile_wide", "tile_deep", "tile_ring", "narrow"])
 @pytest.mark.parametrize("M,H,I", [(1, 256, 128), (50, 2048, 768), (300, 4096, 1408), (2048, 2048, 768)])
 def test_gated_mlp(pra, oracle, variant, M, H, I):
     g = torch.Generator().manual_seed(M + I)

@@ -9,7 +9,7 @@ from _util import bf16_ulp_diff, inputs_mod
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
-VARIANTS = ["stream", "tile_wide", "tile_deep", "narrow"]
+VARIANTS = ["stream", "tile_wide", "tile_deep", "tile_ring", "narrow"]
 
 
 def _problem(oracle, E, k, H, I, M, seed, B=64, routing="softmax"):

@@ -231,7 +231,7 @@ def test_full_size_whole_output_equal_across_families(pra, shape_name, M):
     stream = _run(pra, inp, gemm_variant="stream")
     assert bool(torch.isfinite(stream.float()).all())
     # what the library picks by itself, and both geometries of the LDS-tiled family
-    for variant in ("auto", "tile_wide", "tile_deep"):
+    for variant in ("auto", "tile_wide", "tile_deep", "tile_ring"):
         tiled = _run(pra, inp, gemm_variant=variant)
         differing = int((tiled != stream).sum())
         assert differing == 0, f"{variant}: {differing} of {tiled.numel()} elements differ between the families"
@@ -373,7 +373,7 @@ def test_apply_adapter_and_out_keyword_on_device(pra, oracle):
     (40, 4, 10, 128, "softmax"),      # one row per expert at most
     (16, 2, 1100, 128, "zipf"),
 ])
-@pytest.mark.parametrize("variant", ["tile_wide", "tile_deep"])
+@pytest.mark.parametrize("variant", ["tile_wide", "tile_deep", "tile_ring"])
 def test_tile_list_edge_routings(pra, E, k, M, B, routing, variant):
     im = inputs_mod()
     shape = im.LayerShape("edge", E=E, k=k, H=512, I=512, routing="softmax" if routing == "one_hot" else routing)

@@ -70,7 +70,7 @@ def test_random_shape(pra, oracle, case):
             raise
 
     want = st["cache3"].reshape(P, H)
-    for variant in ("stream", "tile_wide", "tile_deep", "narrow"):
+    for variant in ("stream", "tile_wide", "tile_deep", "tile_ring", "narrow"):
         # a family may support one of the two GEMM shapes of a layer and not the other
         acc1 = attempt(lambda: pra.gemm_acc_i32(x_q, d.w1, s, e, npp, k, B, P, variant))
         acc2 = attempt(lambda: pra.gemm_acc_i32(h_q, d.w2, s, e, npp, 1, B, P, variant))
@@ -83,7 +83,7 @@ def test_random_shape(pra, oracle, case):
         if down is not None:
             assert torch.equal(down.cpu(), want), (variant, int((down.cpu() != want).sum()))
     assert ran >= 1
-    for variant in ("auto", "tile_wide", "tile_deep", "narrow"):
+    for variant in ("auto", "tile_wide", "tile_deep", "tile_ring", "narrow"):
         try:
             out = pra.fused_experts(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, use_int8_w8a8=True,
                                     per_channel_quant=True, w1_scale=d.w1_scale, w2_scale=d.w2_scale,
