@@ -42,7 +42,7 @@ def _profile_traffic(kernel: str, M: int):
     name = "profiles/hbm_traffic_gate_up.txt"
     path = ROOT / name
     if not path.exists():
-        return None
+        return None, None
     for line in path.read_text().splitlines():
         f = line.split()
         if len(f) == 7 and f[0] == "traffic" and f[1] == kernel and f[2] == f"M={M}":
