@@ -62,6 +62,7 @@ struct StreamParams {
   int N;
   int K;
   int B;
+  int64_t cap;        // entries of sorted_ids
   int wave_capacity;  // wavefronts of this kernel the device holds at a time
   int round_even;     // in-kernel quantisation: ties to even instead of away from zero
   void* out;
@@ -103,7 +104,7 @@ __device__ __forceinline__ void pair_rows(const StreamParams& p, int q, int (&wr
 template <int MODE, int NS, bool kFused>
 __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e, int sub0, int first_pair,
                                            int npairs, char* wave_lds, bool count_valid, char* a_lds,
-                                           float* s_lds) {
+                                           float* s_lds, int32_t top_id) {
   const int lane = lane_id();
   const int col = lane & 15;  // token slot inside a sub-tile / weight row inside a tile
   const int grp = lane >> 4;  // which 16 reduction bytes of each step; which 4 output channels
@@ -151,7 +152,11 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
   if (count_valid) {
     for (int base = 0; base < p.B; base += kWave) {
       const int slot = base + lane;
-      const int32_t t = slot < p.B ? p.sorted_ids[(int64_t)blk * p.B + slot] : -1;
+      int32_t t;
+      if (!kFused && base == 0)
+        t = top_id;  // fetched at kernel entry
+      else
+        t = slot < p.B ? p.sorted_ids[(int64_t)blk * p.B + slot] : -1;
       nvalid += __popcll(__ballot(t >= 0 && t < p.P));
     }
   }
@@ -198,7 +203,11 @@ __device__ __forceinline__ int stream_pass(const StreamParams& p, int blk, int e
 #pragma unroll
   for (int s = 0; s < NS; ++s) {
     const int slot = (sub0 + s) * kSub + col;  // a second sub-tile may lie past the end of a small block
-    tok[s] = slot < p.B ? p.sorted_ids[(int64_t)blk * p.B + slot] : -1;
+    if (!kFused && (sub0 + s) * kSub < kWave) {
+      const int32_t early = __shfl(top_id, slot & (kWave - 1));  // one of the first 64 slots: fetched at kernel entry
+      tok[s] = slot < p.B ? early : -1;
+    } else
+      tok[s] = slot < p.B ? p.sorted_ids[(int64_t)blk * p.B + slot] : -1;
     tok_ok[s] = tok[s] >= 0 && tok[s] < p.P;
     const int64_t arow = tok_ok[s] ? tok[s] / p.row_div : 0;
     ap[s] = kFused ? nullptr : p.a_q + arow * K + grp * 16;
@@ -327,7 +336,18 @@ __global__ __launch_bounds__(kThreads, NS == 1 ? 3 : 2) void gemm_stream_kernel(
   __shared__ __align__(16) char lds[kWaves * kWaveLds];
   __shared__ __align__(16) char a_lds[kFused ? kSub * (kFusedMaxK + kFusedRowPad) : 16];
   __shared__ float s_lds[kSub];
+  // Everything that depends only on the position in the grid is requested together with the number of
+  // padded rows, not after it: at kernel entry every such read is a full trip to memory.  (grid.y is the
+  // capacity of the row list in blocks, so these reads are inside the arrays whatever is in use.)
   const int npp = *p.npp;
+  int e_entry = -1;
+  int32_t top_id = -1;
+  if constexpr (!kFused) {
+    e_entry = p.expert_ids[blockIdx.y];
+    const int lane0 = threadIdx.x & (kWave - 1);
+    const int64_t slot0 = (int64_t)blockIdx.y * p.B + lane0;
+    top_id = lane0 < p.B && slot0 < p.cap ? p.sorted_ids[slot0] : -1;
+  }
   const int nblocks = npp / p.B;  // blocks in use: the first ones of the grid's capacity
   const int total_pairs = MODE == kGateUpSilu ? p.N / 2 / 16 : (p.N / 16 + kTiles - 1) / kTiles;
   // Consecutive tile pairs a wavefront streams back to back: one (more wavefronts in flight beat
@@ -355,7 +375,7 @@ __global__ __launch_bounds__(kThreads, NS == 1 ? 3 : 2) void gemm_stream_kernel(
   } else {
     if (blk >= nblocks) return;
   }
-  const int e = p.expert_ids[blk];
+  const int e = kFused ? p.expert_ids[blk] : e_entry;
   if (e < 0 || e >= p.E) return;
   const int first_pair = (group * kWaves + threadIdx.x / kWave) * ppw;
   // a wavefront past the last weight rows leaves, unless the workgroup needs it for the quantisation
@@ -372,15 +392,15 @@ __global__ __launch_bounds__(kThreads, NS == 1 ? 3 : 2) void gemm_stream_kernel(
     if (sub0 * kSub >= p.B) return;
     const int32_t t = p.sorted_ids[(int64_t)blk * p.B + sub0 * kSub];
     if (t < 0 || t >= p.P) return;
-    stream_pass<MODE, NS, kFused>(p, blk, e, sub0, first_pair, npairs, wave_lds, false, a_lds, s_lds);
+    stream_pass<MODE, NS, kFused>(p, blk, e, sub0, first_pair, npairs, wave_lds, false, a_lds, s_lds, top_id);
     return;
   }
   // One workgroup walks all passes; the first one counts the valid rows (a prefix of the block, at
   // least one: the block is in use) to know how many sub-tiles there are.
-  const int nvalid = stream_pass<MODE, NS, kFused>(p, blk, e, 0, first_pair, npairs, wave_lds, true, a_lds, s_lds);
+  const int nvalid = stream_pass<MODE, NS, kFused>(p, blk, e, 0, first_pair, npairs, wave_lds, true, a_lds, s_lds, top_id);
   const int nsub = (nvalid + kSub - 1) / kSub;
   for (int sub0 = NS; sub0 < nsub; sub0 += NS)
-    stream_pass<MODE, NS, kFused>(p, blk, e, sub0, first_pair, npairs, wave_lds, false, a_lds, s_lds);
+    stream_pass<MODE, NS, kFused>(p, blk, e, sub0, first_pair, npairs, wave_lds, false, a_lds, s_lds, top_id);
 }
 
 template <int MODE, bool kFused = false>
@@ -402,6 +422,7 @@ hipError_t launch_mode(const GemmArgs& a, hipStream_t stream) {
   p.K = a.k;
   p.B = a.block_size;
   p.out = a.out;
+  p.cap = a.sorted_cap;
   const int total_pairs = MODE == kGateUpSilu ? a.n / 2 / 16 : (a.n / 16 + kTiles - 1) / kTiles;
   const int waves = total_pairs;  // the kernel groups pairs per wavefront once it knows the blocks in use
   const int64_t blocks = (a.sorted_cap + a.block_size - 1) / a.block_size;
