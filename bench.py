@@ -118,8 +118,8 @@ def time_gate_up_kernel(pkg, torch, shape, dev, weights, steps: int, warmup: int
 
 def time_stages(pkg, torch, shape, dev, weights, steps: int, warmup: int, variant: str) -> list:
     """Every launch of the layer on its own: direct C-ABI calls into preallocated buffers, an event pair per
-    call on the launch stream, with the algorithmic bytes / int8 ops of that launch and the fraction of the
-    roofline that bounds it.  (A launch that does almost nothing still reads about 4 us.  Timed alone back to
+    call on the launch stream (median), with the algorithmic bytes / int8 ops of that launch and the fraction of
+    the roofline that bounds it.  (A launch that does almost nothing still reads about 4 us.  Timed alone back to
     back the gate_up GEMM reads about 10 % above its duration inside the layer, where the memory-bound
     launches around it let the clock recover; the dispatch durations of a kernel trace of the whole layer are
     the in-situ figures.)"""
@@ -167,6 +167,10 @@ def time_stages(pkg, torch, shape, dev, weights, steps: int, warmup: int, varian
         ("moe_sum", lambda i: lib.moe_i8_sum(p_(down), p_(out), M, k, H, stream), 2 * (k + 1) * M * H, 0),
     ]
     result = []
+    # After a stretch of light launches the first dozens of calls of a matrix-bound kernel run through a
+    # transient of the board's power control (first faster, then up to 25 % slower, then steady): every stage
+    # gets at least 40 untimed calls, and the median of the timed ones is reported.
+    warmup = max(warmup, 40)
     for name, fn, nbytes, ops in stages:
         for i in range(warmup):
             abi.check(fn(i))
@@ -177,7 +181,8 @@ def time_stages(pkg, torch, shape, dev, weights, steps: int, warmup: int, varian
             fn(i)
             b.record()
         torch.cuda.synchronize()
-        t = sum(a.elapsed_time(b) for a, b in pairs) / steps * 1e-3
+        times = sorted(a.elapsed_time(b) for a, b in pairs)
+        t = times[len(times) // 2] * 1e-3
         hbm, mfma = nbytes / t / PEAK_HBM_BPS, ops / t / PEAK_INT8_OPS
         result.append({"stage": name, "us": t * 1e6, "bytes": nbytes, "int8_ops": ops, "hbm_frac": hbm,
                        "mfma_frac": mfma, "bound": "mfma" if mfma > hbm else "hbm"})
