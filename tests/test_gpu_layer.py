@@ -53,7 +53,9 @@ def test_fused_experts_full_size_sampled_tokens(pra, oracle, shape_name, M, weig
     out = _run(pra, inp)
     assert bool(torch.isfinite(out.float()).all())
     g = torch.Generator().manual_seed(0)
-    sel = torch.randperm(M, generator=g)[: min(M, 6)].sort()[0]
+    # tokens the oracle recomputes: as many as keep the experts they use (copied to the host) within a few GB
+    weight_bytes = inp.w1.numel() + inp.w2.numel()
+    sel = torch.randperm(M, generator=g)[: min(M, 256 if weight_bytes < (3 << 30) else 32)].sort()[0]
     sub = subset_problem(inp, sel)
     want = oracle.fused_experts(sub["hidden_states"], sub["w1"], sub["w2"], sub["topk_weights"], sub["topk_ids"],
                                 sub["w1_scale"], sub["w2_scale"], 64)
