@@ -68,6 +68,41 @@ __device__ __forceinline__ void wave_histogram(const int (&ids)[kIters], int64_t
   }
 }
 
+// The same placement with the peer masks taken from LDS instead of ballots, for a wavefront that shares its
+// compute unit with fifteen others: there the ~60 vector instructions per 64 pairs that the ballots and the
+// 64-bit per-lane mask arithmetic cost are what bounds the scatter (measured at 8192 pairs in one 1024-thread
+// workgroup: 5.3 of 12.8 us).  Every lane ORs its own bit into a 64-bit word of its expert (`masks`, E words
+// private to the wavefront, zero on entry and on exit); OR does not depend on the order in which the LDS
+// resolves lanes that hit the same word, so the word read back is exactly the ballot-built peer mask.  The
+// lowest lane of a group clears the word and advances the expert's cursor with one LDS atomic whose old value
+// the group picks up by lane permute.  A wavefront's LDS instructions are carried out in program order, which
+// is what makes the read see every lane's OR and keeps the steps of the loop in ascending pair order.
+template <int kIters>
+__device__ __forceinline__ void wave_scatter_masks(const int (&ids)[kIters], int64_t begin, int64_t count, int E,
+                                                   int* cursor, unsigned long long* masks,
+                                                   int32_t* __restrict__ sorted, int64_t sorted_cap) {
+  const int lane = lane_id();
+  const unsigned long long my_bit = 1ull << lane;
+#pragma unroll
+  for (int i = 0; i < kIters; ++i) {
+    if ((int64_t)i * kWave >= count) break;
+    const int e = ids[i];
+    const bool active = e >= 0 && e < E;
+    if (active) atomicOr(masks + e, my_bit);
+    __builtin_amdgcn_wave_barrier();
+    const unsigned long long peers = active ? masks[e] : my_bit;
+    __builtin_amdgcn_wave_barrier();
+    const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(peers >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)peers, 0u));
+    int first = 0;
+    if (active && rank == 0) {
+      masks[e] = 0ull;
+      first = atomicAdd(cursor + e, __popcll(peers));
+    }
+    const int pos = __shfl(first, __ffsll(peers) - 1) + rank;
+    if (active && pos < sorted_cap) sorted[pos] = (int32_t)(begin + i * kWave + lane);
+  }
+}
+
 // sorted[cursor[x]++] = pair index, in ascending pair index per expert.
 template <int kIters>
 __device__ __forceinline__ void wave_scatter(const int (&ids)[kIters], int64_t begin, int64_t count, int E,
@@ -130,18 +165,27 @@ __device__ __forceinline__ void write_expert_ids(const int* seg, int E, int B, i
   }
 }
 
-// LDS layout: hist[kSingleWaves][E] | seg[E + 1] | wave_sums[kSingleWaves + 1]
+// Ints of LDS in front of the peer-mask words, a multiple of two so that those are 8-byte aligned.
+__host__ __device__ constexpr size_t single_lds_ints(int E) {
+  return ((size_t)kSingleWaves * E + E + 1 + kSingleWaves + 1 + 1) / 2 * 2;
+}
+
+// LDS layout: hist[kSingleWaves][E] | seg[E + 1] | wave_sums[kSingleWaves + 1] | with `use_masks`:
+// peer masks[kSingleWaves][E] (64-bit)
 __device__ __forceinline__ void align_single_body(
     const int32_t* __restrict__ ids, int P, int E, int B, int nbits,
     int32_t* __restrict__ sorted, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
-    int64_t expert_cap, int32_t* __restrict__ npp_out, int* smem) {
+    int64_t expert_cap, int32_t* __restrict__ npp_out, int* smem, bool use_masks) {
   int* hist = smem;
   int* seg = hist + kSingleWaves * E;
   int* wave_sums = seg + E + 1;
+  unsigned long long* masks = reinterpret_cast<unsigned long long*>(smem + single_lds_ints(E));
   const int tid = threadIdx.x;
   const int wave = tid / kWave;
 
   for (int i = tid; i < kSingleWaves * E; i += kSingleThreads) hist[i] = 0;
+  if (use_masks)
+    for (int i = tid; i < kSingleWaves * E; i += kSingleThreads) masks[i] = 0ull;
   for (int64_t i = tid; i < sorted_cap; i += kSingleThreads) sorted[i] = P;
   __syncthreads();
 
@@ -175,15 +219,18 @@ __device__ __forceinline__ void align_single_body(
     for (int w = 0; w < kSingleWaves; ++w) hist[w * E + tid] += start;
   write_expert_ids(seg, E, B, npp, expert_ids, expert_cap);
   __syncthreads();
-  wave_scatter(mine, begin, end - begin, E, nbits, hist + wave * E, sorted, sorted_cap);
+  if (use_masks)
+    wave_scatter_masks(mine, begin, end - begin, E, hist + wave * E, masks + wave * E, sorted, sorted_cap);
+  else
+    wave_scatter(mine, begin, end - begin, E, nbits, hist + wave * E, sorted, sorted_cap);
 }
 
 __global__ __launch_bounds__(kSingleThreads) void align_single_kernel(
     const int32_t* __restrict__ ids, int P, int E, int B, int nbits,
     int32_t* __restrict__ sorted, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
-    int64_t expert_cap, int32_t* __restrict__ npp_out) {
+    int64_t expert_cap, int32_t* __restrict__ npp_out, int use_masks) {
   extern __shared__ int smem[];
-  align_single_body(ids, P, E, B, nbits, sorted, sorted_cap, expert_ids, expert_cap, npp_out, smem);
+  align_single_body(ids, P, E, B, nbits, sorted, sorted_cap, expert_ids, expert_cap, npp_out, smem, use_masks != 0);
 }
 
 // One launch for small batches: workgroup 0 runs moe_align, every other workgroup quantises 16
@@ -192,10 +239,10 @@ template <int VPL>
 __global__ __launch_bounds__(kSingleThreads) void align_quant_kernel(
     const int32_t* __restrict__ ids, int P, int E, int B, int nbits,
     int32_t* __restrict__ sorted, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
-    int64_t expert_cap, int32_t* __restrict__ npp_out, QuantArgs q) {
+    int64_t expert_cap, int32_t* __restrict__ npp_out, int use_masks, QuantArgs q) {
   extern __shared__ int smem[];
   if (blockIdx.x == 0) {
-    align_single_body(ids, P, E, B, nbits, sorted, sorted_cap, expert_ids, expert_cap, npp_out, smem);
+    align_single_body(ids, P, E, B, nbits, sorted, sorted_cap, expert_ids, expert_cap, npp_out, smem, use_masks != 0);
     return;
   }
   const int64_t row = (int64_t)(blockIdx.x - 1) * kSingleWaves + threadIdx.x / kWave;
@@ -475,6 +522,12 @@ bool align_quant_fusable(const AlignArgs& a, const QuantArgs& q) {
 
 namespace {
 size_t single_lds_bytes(int E) { return sizeof(int) * ((size_t)kSingleWaves * E + E + 1 + kSingleWaves + 1); }
+// The single-workgroup kernel with its peer masks in LDS: used while they fit beside the histograms and while
+// there is more than one 64-pair step per wavefront to rank (otherwise there is nothing to gain).
+constexpr int kMaskMaxExperts = 256;
+bool single_uses_masks(int E, int64_t num_pairs) { return E <= kMaskMaxExperts && num_pairs > kSingleWaves * kWave; }
+size_t single_masks_lds_bytes(int E) { return sizeof(int) * single_lds_ints(E) + sizeof(unsigned long long) * kSingleWaves * (size_t)E; }
+constexpr int kSingleMasksLdsMax = (int)(sizeof(int) * single_lds_ints(kMaskMaxExperts) + sizeof(unsigned long long) * kSingleWaves * (size_t)kMaskMaxExperts);
 constexpr int kSingleLdsMax = (int)(sizeof(int) * ((size_t)kSingleWaves * kMaxExperts + kMaxExperts + kSingleWaves + 2));
 
 // The kernels of the two-launch path may need more dynamic LDS than the default limit (1024 experts).
@@ -565,16 +618,18 @@ hipError_t launch_align_quant(const AlignArgs& a, const QuantArgs& q, hipStream_
                        a.sorted_cap);
     return hipGetLastError();
   }
+  const bool use_masks = single_uses_masks(E, a.num_pairs);
+  const size_t lds_bytes = use_masks ? single_masks_lds_bytes(E) : single_lds_bytes(E);
 #define MOE_I8_FUSED_LAUNCH(V)                                                                      \
   do {                                                                                              \
-    static const hipError_t attr = hipFuncSetAttribute((const void*)align_quant_kernel<V>,          \
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize,  \
-                                                       kSingleLdsMax);                              \
+    static const hipError_t attr = hipFuncSetAttribute(                                             \
+        (const void*)align_quant_kernel<V>, hipFuncAttributeMaxDynamicSharedMemorySize,             \
+        kSingleLdsMax > kSingleMasksLdsMax ? kSingleLdsMax : kSingleMasksLdsMax);                   \
     if (attr != hipSuccess) return attr;                                                            \
-    hipLaunchKernelGGL(align_quant_kernel<V>, grid, dim3(kSingleThreads), single_lds_bytes(E),      \
+    hipLaunchKernelGGL(align_quant_kernel<V>, grid, dim3(kSingleThreads), lds_bytes,                \
                        stream, a.topk_ids, (int)a.num_pairs, E, a.block_size, bits_for(E),          \
                        a.sorted_token_ids, a.sorted_cap, a.expert_ids, a.expert_cap,                \
-                       a.num_tokens_post_padded, q);                                                \
+                       a.num_tokens_post_padded, use_masks ? 1 : 0, q);                             \
   } while (0)
   switch (quant_vectors_per_lane(q.cols)) {
     case 1: MOE_I8_FUSED_LAUNCH(1); break;
@@ -591,14 +646,15 @@ hipError_t launch_align(const AlignArgs& a, hipStream_t stream) {
   const int E = a.num_experts;
   const int nbits = bits_for(E);
   if (a.num_pairs <= kSingleMaxPairs) {
-    const size_t lds = sizeof(int) * ((size_t)kSingleWaves * E + E + 1 + kSingleWaves + 1);
+    const bool use_masks = single_uses_masks(E, a.num_pairs);
+    const size_t lds = use_masks ? single_masks_lds_bytes(E) : single_lds_bytes(E);
     static const hipError_t attr = hipFuncSetAttribute(
         (const void*)align_single_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-        (int)(sizeof(int) * ((size_t)kSingleWaves * kMaxExperts + kMaxExperts + kSingleWaves + 2)));
+        kSingleLdsMax > kSingleMasksLdsMax ? kSingleLdsMax : kSingleMasksLdsMax);
     if (attr != hipSuccess) return attr;
     hipLaunchKernelGGL(align_single_kernel, dim3(1), dim3(kSingleThreads), lds, stream, a.topk_ids,
                        (int)a.num_pairs, E, a.block_size, nbits, a.sorted_token_ids, a.sorted_cap,
-                       a.expert_ids, a.expert_cap, a.num_tokens_post_padded);
+                       a.expert_ids, a.expert_cap, a.num_tokens_post_padded, use_masks ? 1 : 0);
     return hipGetLastError();
   }
   if (a.num_pairs <= kChunkedMaxPairs) {
